@@ -1,0 +1,202 @@
+"""Pins for the CPU oracle that do not involve the reference at all: closed forms, brute force,
+and library routines (torch on CPU).  Each one is chosen so that a plausible slip -- a transposed
+operand, a wrong tap order, eps inside the root, a swapped gate -- fails it."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import binding as ob
+
+
+def rel(a, b):
+    return float(np.abs(a.astype(np.float64) - b.astype(np.float64)).max() / max(np.abs(b).max(), 1e-30))
+
+
+def test_im2col_closed_form_bruteforce():
+    rng = np.random.default_rng(0)
+    for (c, h, w, k, s, p) in [(2, 6, 7, 3, 1, 1), (3, 9, 9, 5, 2, 2), (1, 11, 11, 11, 4, 0), (2, 5, 5, 2, 2, 1)]:
+        im = rng.standard_normal((c, h, w)).astype(np.float32)
+        col = ob.im2col(im, k, s, p)
+        oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+        assert col.shape == (c * k * k, oh * ow)
+        for ci in range(c):
+            for i in range(k):
+                for j in range(k):
+                    for y in range(oh):
+                        for x in range(ow):
+                            yy, xx = y * s + i - p, x * s + j - p
+                            want = im[ci, yy, xx] if 0 <= yy < h and 0 <= xx < w else 0.0
+                            assert col[(ci * k + i) * k + j, y * ow + x] == want
+
+
+@pytest.mark.parametrize("geom", [(2, 3, 12, 12, 5, 3, 1, 1), (2, 4, 15, 13, 6, 5, 2, 2), (1, 3, 23, 23, 4, 11, 4, 0),
+                                  (3, 8, 7, 7, 16, 1, 1, 0), (2, 3, 14, 14, 4, 7, 2, 3)])
+def test_conv_equals_cross_correlation(geom):
+    B, Cc, H, W, Fo, k, s, p = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Fo, Cc, k, k)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(Fo).astype(np.float32)
+    got = ob.conv_forward(x, w, b, None, s, p, "linear")
+    want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(b).double(),
+                    stride=s, padding=p).numpy()
+    assert got.shape == want.shape
+    assert rel(got, want) < 1e-5
+
+
+def test_conv_bn_is_affine_with_eps_outside_root():
+    # y = bias + scale * (conv - mean) / (sqrt(var) + 1e-5); a small variance makes eps placement visible
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((2, 3, 8, 8)).astype(np.float32)
+    w = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    bias = rng.standard_normal(4).astype(np.float32)
+    scale = rng.uniform(0.8, 1.2, 4).astype(np.float32)
+    mean = (rng.standard_normal(4) * 0.1).astype(np.float32)
+    var = np.array([1e-6, 4e-6, 1.0, 0.5], np.float32)
+    got = ob.conv_forward(x, w, bias, (scale, mean, var), 1, 1, "linear").astype(np.float64)
+    raw = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), None, padding=1).numpy()
+    sh = (1, 4, 1, 1)
+    outside = (raw - mean.reshape(sh)) / (np.sqrt(var.astype(np.float64)).reshape(sh) + 1e-5) * scale.reshape(sh) \
+        + bias.reshape(sh)
+    inside = (raw - mean.reshape(sh)) / np.sqrt(var.astype(np.float64) + 1e-5).reshape(sh) * scale.reshape(sh) \
+        + bias.reshape(sh)
+    assert rel(got, outside) < 1e-5
+    assert rel(got, inside) > 1e-2      # the other placement is far away for var ~ 1e-6
+
+
+def test_connected_is_x_times_w_transposed():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((7, 3, 4, 5)).astype(np.float32)     # NCHW flatten
+    w = rng.standard_normal((11, 60)).astype(np.float32)
+    b = rng.standard_normal(11).astype(np.float32)
+    got = ob.connected_forward(x, w, b, None, "linear")
+    want = x.reshape(7, 60).astype(np.float64) @ w.astype(np.float64).T + b
+    assert rel(got, want) < 1e-5
+
+
+def test_maxpool_equals_torch_when_window_equals_stride():
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((2, 3, 12, 12)).astype(np.float32)
+    y, idx = ob.maxpool_forward(x, 2, 2, 0)
+    ty, tidx = F.max_pool2d(torch.from_numpy(x), 2, 2, return_indices=True)
+    np.testing.assert_array_equal(y, ty.numpy())
+    # torch indexes within one (b, c) plane; the reference stores the offset into the whole tensor
+    plane = np.arange(6).reshape(2, 3, 1, 1) * 144
+    np.testing.assert_array_equal(idx, (tidx.numpy() + plane).astype(np.uint32))
+    # and the index really addresses the maximum
+    np.testing.assert_array_equal(x.ravel()[idx.ravel()], y.ravel())
+
+
+def test_maxpool_k3s2_and_size_rule():
+    # AlexNet chain 55 -> 27 -> 13 -> 6 with padding 0 and ResNet 112 -> 56 (out = (in + 2p) / stride)
+    assert [ob.pool_out_dim(n, 2, 0) for n in (55, 27, 13, 112)] == [27, 13, 6, 56]
+    assert ob.oracle().orc_pool_default_padding(3) == 1 and ob.oracle().orc_pool_default_padding(2) == 0
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((1, 2, 11, 11)).astype(np.float32)
+    y, idx = ob.maxpool_forward(x, 3, 2, 0)      # 11 -> 5, every window inside the image
+    ty = F.max_pool2d(torch.from_numpy(x), 3, 2)
+    np.testing.assert_array_equal(y, ty.numpy())
+    # first maximum wins on ties (row-major scan of the window)
+    x2 = np.zeros((1, 1, 4, 4), np.float32)
+    _, idx2 = ob.maxpool_forward(x2, 2, 2, 0)
+    np.testing.assert_array_equal(idx2.ravel(), [0, 2, 8, 10])
+
+
+def test_avgpool_counts_padding():
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 2, 8, 8)).astype(np.float32)
+    got = ob.avgpool_forward(x, 3, 2, 1)        # (8 + 2) / 2 = 5 outputs; the last window hangs off the edge
+    padded = np.zeros((2, 2, 12, 12), np.float64)
+    padded[:, :, 1:9, 1:9] = x
+    want = np.zeros((2, 2, 5, 5))
+    for h in range(5):
+        for w in range(5):
+            want[:, :, h, w] = padded[:, :, 2 * h:2 * h + 3, 2 * w:2 * w + 3].sum(axis=(2, 3)) / 9.0
+    assert rel(got, want) < 1e-6
+    glob = ob.avgpool_forward(x[:, :, :7, :7], 7, 7, 0)
+    assert rel(glob.reshape(2, 2), x[:, :, :7, :7].astype(np.float64).mean(axis=(2, 3))) < 1e-6
+
+
+def test_shortcut_invariants():
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((2, 4, 6, 6)).astype(np.float32)
+    b = rng.standard_normal((2, 4, 6, 6)).astype(np.float32)
+    np.testing.assert_array_equal(ob.shortcut_forward(b, a), a + b)           # same shape: plain add
+    wide = rng.standard_normal((2, 16, 6, 6)).astype(np.float32)
+    out = ob.shortcut_forward(wide, a)                                         # channel growth
+    np.testing.assert_array_equal(out[:, :4], wide[:, :4] + a)
+    np.testing.assert_array_equal(out[:, 4:], wide[:, 4:])
+    small = rng.standard_normal((2, 8, 3, 3)).astype(np.float32)
+    out = ob.shortcut_forward(small, a)                                        # 6 -> 3: conn[::2, ::2]
+    np.testing.assert_array_equal(out[:, :4], small[:, :4] + a[:, :, ::2, ::2])
+    odd = rng.standard_normal((1, 2, 19, 19)).astype(np.float32)
+    tgt = rng.standard_normal((1, 2, 10, 10)).astype(np.float32)
+    out = ob.shortcut_forward(tgt, odd)                                        # 19 / 10 = 1: top-left crop
+    np.testing.assert_array_equal(out, tgt + odd[:, :, :10, :10])
+    relu = ob.shortcut_forward(b, a, "relu")
+    np.testing.assert_array_equal(relu, np.maximum(a + b, 0))
+
+
+def test_softmax_properties():
+    rng = np.random.default_rng(10)
+    x = (rng.standard_normal((5, 1000)) * 4).astype(np.float32)
+    y = ob.softmax_forward(x)
+    assert np.abs(y.sum(axis=1) - 1).max() < 1e-5
+    assert rel(y, torch.softmax(torch.from_numpy(x).double(), 1).numpy()) < 1e-5
+    shifted = ob.softmax_forward(x + np.float32(8.0))
+    assert rel(shifted, y) < 1e-5
+    assert (y.argmax(1) == x.argmax(1)).all()
+
+
+def test_activation_closed_forms():
+    x = np.linspace(-6, 6, 2001).astype(np.float32)
+    d = x.astype(np.float64)
+    assert rel(ob.activate("logistic", x), 1 / (1 + np.exp(-d))) < 1e-6
+    assert rel(ob.activate("tanh", x), np.tanh(d)) < 1e-6
+    assert rel(ob.activate("loggy", x), 2 / (1 + np.exp(-d)) - 1) < 1e-6
+    np.testing.assert_array_equal(ob.activate("relu", x), np.maximum(x, 0))
+    np.testing.assert_array_equal(ob.activate("leaky", x), np.where(x > 0, x, (0.1 * d).astype(np.float32)))
+    np.testing.assert_array_equal(ob.activate("relie", x), np.where(x > 0, x, (0.01 * d).astype(np.float32)))
+    np.testing.assert_array_equal(ob.activate("linear", x), x)
+    # the three that differ from the textbook: squares, and 0/1 indicators
+    np.testing.assert_array_equal(ob.activate("elu", x)[x > 0], (x * x)[x > 0])
+    np.testing.assert_array_equal(ob.activate("hardtan", x), ((x > -1) & (x < 1)).astype(np.float32))
+    np.testing.assert_array_equal(ob.activate("lhtan", x), ((x > 0) & (x < 1)).astype(np.float32))
+
+
+def test_lstm_equals_torch_lstm():
+    # standard cell, two bias vectors, no peepholes.  File order iW,fW,oW,cW,iU,fU,oU,cU; torch packs i,f,g,o.
+    rng = np.random.default_rng(12)
+    T, B, I, H = 5, 3, 7, 6
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    names = ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU")
+    wt = {n: (rng.standard_normal((H, H if n[1] == "W" else I)) * 0.4).astype(np.float32) for n in names}
+    bs = {n: (rng.standard_normal(H) * 0.3).astype(np.float32) for n in names}
+    y, cell = ob.lstm_forward(x, [wt[n] for n in names], [bs[n] for n in names], want_cell=True)
+    lstm = torch.nn.LSTM(I, H).double()
+    with torch.no_grad():
+        lstm.weight_ih_l0.copy_(torch.from_numpy(np.concatenate([wt["iU"], wt["fU"], wt["cU"], wt["oU"]])))
+        lstm.weight_hh_l0.copy_(torch.from_numpy(np.concatenate([wt["iW"], wt["fW"], wt["cW"], wt["oW"]])))
+        lstm.bias_ih_l0.copy_(torch.from_numpy(np.concatenate([bs["iU"], bs["fU"], bs["cU"], bs["oU"]])))
+        lstm.bias_hh_l0.copy_(torch.from_numpy(np.concatenate([bs["iW"], bs["fW"], bs["cW"], bs["oW"]])))
+        ty, (hn, cn) = lstm(torch.from_numpy(x).double())
+    assert rel(y, ty.numpy()) < 1e-5
+    assert rel(cell[-1], cn[0].numpy()) < 1e-5
+
+
+def test_openblas_backend_matches_custom_gemm():
+    if not ob.use_openblas(threads=2):
+        pytest.skip("no OpenBLAS found")
+    try:
+        rng = np.random.default_rng(13)
+        x = rng.standard_normal((2, 5, 14, 14)).astype(np.float32)
+        w = (rng.standard_normal((7, 5, 3, 3)) * 0.2).astype(np.float32)
+        b = rng.standard_normal(7).astype(np.float32)
+        fast = ob.conv_forward(x, w, b, None, 1, 1, "relu")
+        ob.use_custom_gemm()
+        slow = ob.conv_forward(x, w, b, None, 1, 1, "relu")
+        assert rel(fast, slow) < 1e-5
+    finally:
+        ob.use_custom_gemm()
+        ob.set_threads(1)
