@@ -1,0 +1,177 @@
+/*
+ * nebula_hip.h -- C ABI of the MI355X (gfx950) forward path for Nebula's layer framework.
+ *
+ * One shared library (libnebula_hip.so) exports these entry points.  They take plain pointers and
+ * sizes, return an int status (0 = NBL_OK) and never throw.  Every entry point names the interface
+ * of the reference (yonseicasl/Nebula v1.4.1, paths relative to its tree) that it stands in for.
+ *
+ * Conventions (the reference's own, models/layers/layer.h:41-70):
+ *   - tensors are fp32, NCHW, row-major, batch outermost; conv weights OIHW; FC weights [O][I];
+ *     recurrent tensors are time-major [T][B][feature];
+ *   - activation ids are the reference's activation_type_t values (common/def.h:62-78);
+ *   - pointers named *_dev are device pointers valid on the context's GPU, pointers named *_host are
+ *     host pointers; the caller owns every buffer it passes in;
+ *   - all work is queued on the context's stream and is asynchronous; nbl_sync() waits for it.
+ *     A context is not thread-safe.  Results follow the reference's CPU (.cc) path where its CPU
+ *     and CUDA paths disagree.
+ */
+#ifndef NEBULA_HIP_H
+#define NEBULA_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nbl_ctx nbl_ctx;
+typedef struct nbl_conv_plan nbl_conv_plan;
+typedef struct nbl_fc_plan nbl_fc_plan;
+typedef struct nbl_lstm_plan nbl_lstm_plan;
+
+enum nbl_status {
+    NBL_OK = 0,
+    NBL_EINVAL = -1,        /* bad argument (null pointer, zero size, unknown id, shape mismatch) */
+    NBL_EHIP = -2,          /* a HIP runtime call failed; nbl_last_error() has its text */
+    NBL_ENOMEM = -3,        /* device allocation failed */
+    NBL_EUNSUPPORTED = -4,  /* valid request outside what the kernels cover (e.g. > 2^31 elements) */
+    NBL_ENODEVICE = -5      /* no usable gfx950 device */
+};
+
+/* activation_type_t, common/def.h:62-78 */
+enum nbl_activation {
+    NBL_ACT_UNDEFINED = 0, NBL_ACT_ELU, NBL_ACT_HARDTAN, NBL_ACT_LEAKY, NBL_ACT_LHTAN, NBL_ACT_LINEAR,
+    NBL_ACT_LOGGY, NBL_ACT_LOGISTIC, NBL_ACT_PLSE, NBL_ACT_RAMP, NBL_ACT_RELIE, NBL_ACT_RELU,
+    NBL_ACT_STAIR, NBL_ACT_TANH, NBL_ACT_COUNT
+};
+
+enum nbl_pool_mode { NBL_POOL_MAX = 0, NBL_POOL_AVG = 1 };
+
+/* ---- context, memory, stream -------------------------------------------------------------------
+ * Replaces network_t's constructor state: cudaSetDevice(0) + cublasCreate/cudnnCreate
+ * (models/networks/network.cc:43-51) and the bare cudaMalloc/cudaMemcpy/cudaMemset calls spread over
+ * every layer's init()/init_weight() (e.g. models/layers/convolutional_layer.cc:186-229,335-347). */
+int nbl_ctx_create(int device, nbl_ctx **out);
+/* Same, but queue all work on an existing hipStream_t (passed as void*); NULL = the null stream. */
+int nbl_ctx_create_on_stream(int device, void *hip_stream, nbl_ctx **out);
+int nbl_ctx_destroy(nbl_ctx *ctx);
+/* Text of the last failure on this context ("" if none); with ctx == NULL, of the last failed
+ * nbl_ctx_create*.  The string stays valid until the next failing call. */
+const char *nbl_last_error(nbl_ctx *ctx);
+void *nbl_ctx_stream(nbl_ctx *ctx);
+int nbl_malloc(nbl_ctx *ctx, void **dev_ptr, size_t bytes);
+int nbl_free(nbl_ctx *ctx, void *dev_ptr);
+int nbl_h2d(nbl_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);   /* returns after the copy */
+int nbl_d2h(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);   /* returns after the copy */
+int nbl_fill_zero(nbl_ctx *ctx, void *dst_dev, size_t bytes);                   /* a fill kernel, capturable */
+int nbl_sync(nbl_ctx *ctx);
+
+/* ---- convolution -------------------------------------------------------------------------------
+ * nbl_conv2d_pack replaces convolutional_layer_t::init_weight()'s upload
+ * (models/layers/convolutional_layer.cc:257-260,312-316,335-347): it takes the HOST arrays exactly as
+ * they sit in the .wgh file (bias[F], weight[F][C][k][k], and scale/rolling_mean/rolling_variance[F]
+ * or three NULLs when batch_normalize=0), re-lays the weights out for the implicit-GEMM kernel and
+ * turns inference batchnorm + bias into one per-filter multiply-add
+ *     y = act(conv * g + b),  g = scale / (sqrt(var) + 1e-5),  b = bias - mean * g
+ * (the CPU form, common/batchnorm.cc:70: eps outside the root).
+ *
+ * nbl_conv2d_fwd replaces convolutional_layer_t::_forward_() (models/layers/convolutional_layer.cu:11-84;
+ * CPU twin convolutional_layer.cc:365-409): per-image _im2col_ + cublasSgemm, _forward_batchnorm_,
+ * _forward_bias_, _activate_ become one kernel.  x_dev [B][C][H][W] -> y_dev [B][F][OH][OW],
+ * OH = (H + 2*pad - k)/stride + 1. */
+int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
+                    const float *scale_host, const float *mean_host, const float *var_host,
+                    unsigned C, unsigned H, unsigned W, unsigned F,
+                    unsigned ksize, unsigned stride, unsigned pad, int act, nbl_conv_plan **out);
+int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B);
+int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *plan);
+/* Algorithmic FLOP of one forward at batch B (2*B*F*OH*OW*C*k*k) and the output dims. */
+int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, double *flop_per_image);
+/* Pick the tile shape by hand (tests / tuning); variant < 0 restores the built-in choice.
+ * nbl_conv2d_num_variants() says how many exist. */
+int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
+int nbl_conv2d_num_variants(void);
+
+/* Replaces _im2col_ (common/utils.h:48, utils.cu:34-74; CPU twin utils.cc:81-119).  The convolution
+ * kernel never writes this buffer; the entry point exists so the gather it performs on the fly
+ * (same device function, same index table) can be checked element for element.
+ * x_dev [C][H][W] (one image) -> col_dev [C*k*k][OH*OW]. */
+int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigned W,
+               unsigned ksize, unsigned stride, unsigned pad, float *col_dev);
+
+/* ---- fully connected ---------------------------------------------------------------------------
+ * nbl_fc_pack: connected_layer_t::init_weight() (models/layers/connected_layer.cc:186-206); HOST
+ * arrays in .wgh order bias[O], weight[O][I], [scale, mean, var][O] or NULLs.
+ * nbl_fc_fwd: connected_layer_t::_forward_() (models/layers/connected_layer.cu:19-53; CPU twin
+ * connected_layer.cc:245-277): y[B][O] = act((x[B][I] . W^T) * g + b).  (The CUDA file adds bias[0]
+ * to every output, connected_layer.cu:44; the CPU file is followed.) */
+int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
+                const float *scale_host, const float *mean_host, const float *var_host,
+                unsigned I, unsigned O, int act, nbl_fc_plan **out);
+int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B);
+int nbl_fc_plan_destroy(nbl_ctx *ctx, nbl_fc_plan *plan);
+
+/* ---- LSTM --------------------------------------------------------------------------------------
+ * nbl_lstm_pack: lstm_layer_t::init_weight() (models/layers/lstm_layer.cc:194-206).  The eight
+ * sub-layers come as HOST arrays in FILE order iW, fW, oW, cW, iU, fU, oU, cU: weight_host[s] is
+ * [H][H] for the W (hidden) four and [H][I] for the U (input) four, bias_host[s] is [H];
+ * scale/mean/var_host are arrays of eight [H] vectors, or NULL when batch_normalize=0.
+ * sub_act is the [lstm] section's activation, which the reference applies inside every sub-layer.
+ * nbl_lstm_fwd: lstm_layer_t::_forward_() (models/layers/lstm_layer.cu:15-140; CPU twin
+ * lstm_layer.cc:233-346) from zero hidden and cell state: x_dev [T][B][I] -> y_dev [T][B][H].
+ * The per-step 8 GEMMs + 5 saxpy + 7 copies + 7 elementwise kernels become one input-side GEMM over
+ * all steps and one fused recurrent kernel per step.  cell_dev (optional, may be NULL) receives the
+ * final cell state [B][H]. */
+int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *const *bias_host,
+                  const float *const *scale_host, const float *const *mean_host, const float *const *var_host,
+                  unsigned I, unsigned H, int sub_act, nbl_lstm_plan **out);
+int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *plan, const float *x_dev, float *y_dev, float *cell_dev,
+                 unsigned T, unsigned B);
+int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *plan);
+
+/* ---- memory-bound layers -----------------------------------------------------------------------
+ * nbl_pool_fwd: pooling_layer_t::_forward_() (models/layers/pooling_layer.cu:150-172; CPU twin
+ * pooling_layer.cc:109-182).  Output size is the reference's rule OH = (H + 2*pad)/stride.
+ * Max: first maximum in row-major window order wins, taps outside the image count as -1e8, index_dev
+ * (may be NULL) receives the flat offset into the whole input tensor (0xffffffff if nothing beat the
+ * sentinel).  Avg: sum of the in-image taps divided by k*k. */
+int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index_dev,
+                 unsigned B, unsigned C, unsigned H, unsigned W,
+                 unsigned ksize, unsigned stride, unsigned pad, int mode);
+unsigned nbl_pool_out_dim(unsigned in, unsigned stride, unsigned pad);
+unsigned nbl_conv_out_dim(unsigned in, unsigned ksize, unsigned stride, unsigned pad);
+
+/* shortcut_layer_t::_forward_() (models/layers/shortcut_layer.cu:27-52; CPU twin
+ * shortcut_layer.cc:68-79 + common/utils.cc:28-60): y = act(prev + strided/cropped conn).
+ * prev_dev and y_dev are [B][out_c][out_h][out_w] (y_dev may alias prev_dev); conn_dev is
+ * [B][in_c][in_h][in_w]. */
+int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev, float *y_dev, unsigned B,
+                     unsigned in_c, unsigned in_h, unsigned in_w,
+                     unsigned out_c, unsigned out_h, unsigned out_w, int act);
+
+/* softmax_layer_t::_forward_() (models/layers/softmax_layer.cu:30-41; CPU twin softmax_layer.cc:85-106). */
+int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned rows, unsigned n);
+
+/* layer_t::_activate_() and the 13 _<name>_activation_ functions (models/layers/layer.cu:9-69,
+ * common/activations.h:38-50; CPU twins common/activations.cc:6-89), in place. */
+int nbl_activation_fwd(nbl_ctx *ctx, float *x_dev, size_t n, int act);
+
+/* _forward_bias_ (common/utils.h:55; CPU twin utils.cc:162-179): y[b][c][s] += bias[c]. */
+int nbl_forward_bias(nbl_ctx *ctx, float *y_dev, const float *bias_dev,
+                     unsigned channel, unsigned size, unsigned batch);
+/* _batchnorm_normalize_ + _batchnorm_scale_down_ (common/batchnorm.h:31-33; CPU twins
+ * batchnorm.cc:58-97): y = (y - mean[c]) / (sqrt(var[c]) + 1e-5) * scale[c], in place. */
+int nbl_batchnorm_inference(nbl_ctx *ctx, float *y_dev, const float *mean_dev, const float *var_dev,
+                            const float *scale_dev, unsigned channel, unsigned size, unsigned batch);
+
+/* ---- timing ------------------------------------------------------------------------------------
+ * HIP-event timing on the context's own stream (torch.cuda.Event would watch torch's stream). */
+int nbl_timer_start(nbl_ctx *ctx);
+int nbl_timer_stop(nbl_ctx *ctx, float *elapsed_ms);   /* waits for the stop event */
+
+const char *nbl_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,464 @@
+// C[m][n] = sum_k A[m][k] * Bw[n][k]  ("NT": both operands k-contiguous) on the fp32 matrix cores,
+// with the epilogues of the fully-connected layer and of the LSTM cell.
+//
+// Fully connected (models/layers/connected_layer.cc:245-277): A = activations [B][I], Bw = the weight
+// matrix exactly as the .wgh file holds it, [O][I].  Batch rows are the MFMA rows and output neurons
+// the MFMA columns, so one accumulator row is written as 32 consecutive floats of y[b][:].
+//
+// LSTM (models/layers/lstm_layer.cc:233-346): the input half  U.x  is hoisted out of the time loop
+// (one GEMM over all T*B rows) and the recurrent half  W.h  runs once per step with the gate
+// non-linearities and the cell update in its epilogue.  The four gate matrices are interleaved at
+// pack time in blocks of 32 hidden units, so that the four 32x32 accumulators a wave owns are the
+// i, f, g, o pre-activations of the same (batch row, hidden unit) elements and the whole cell update
+// happens in registers.
+//
+// LDS layout: [row][BK + 4] floats per operand.  A k-tile of 32 is consumed by 16 MFMAs; lanes 0-31
+// feed k = 0..15 and lanes 32-63 feed k = 16..31 (any pairing of k values is legal as long as both
+// operands use the same one), so every lane fetches its 16 values as four 16-byte LDS reads.
+#include "nbl_internal.h"
+
+#include <cmath>
+#include <vector>
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int GEMM_BK = 32;
+constexpr int GEMM_LD = GEMM_BK + 4;
+
+enum { EPI_DIRECT = 0, EPI_PARTIAL = 1, EPI_LSTM = 2 };
+
+struct GemmArgs {
+    const float *A; const float *Bw; float *C;
+    int M, N, K, lda, ldb, ldc;
+    int vec_ok;               // rows 16-byte aligned and K % 4 == 0: float4 global loads are legal
+    int k_chunk;              // k range per blockIdx.z (multiple of GEMM_BK)
+    // EPI_DIRECT: C = act((acc * g[n]) + b[n])
+    const float *g; const float *b; int act, has_scale;
+    // EPI_LSTM: N = 4*Hp in interleaved order; gx [M][N] input-side pre-activations (already activated by
+    // sub_act), b = recurrent-side bias, act = sub_act; c [M][H] cell state (in place), C = h out [M][H]
+    const float *gx; float *c; int H;
+};
+
+__device__ __forceinline__ float4 load_row4(const float *__restrict__ base, int row, int rows, int ld,
+                                            int k, int K, int vec_ok) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if(row < rows) {
+        const float *p = base + (size_t)row * ld + k;
+        if(vec_ok && k + 3 < K) {
+            v = *reinterpret_cast<const float4*>(p);
+        } else {
+            if(k < K) v.x = p[0];
+            if(k + 1 < K) v.y = p[1];
+            if(k + 2 < K) v.z = p[2];
+            if(k + 3 < K) v.w = p[3];
+        }
+    }
+    return v;
+}
+
+template<int MT, int NT, int WAVES_M, int WAVES_N, int EPI>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N)
+void gemm_nt_kernel(const GemmArgs a) {
+    constexpr int BK = GEMM_BK, LD = GEMM_LD;
+    constexpr int NTHREADS = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = MT * 32 * WAVES_M, BN = NT * 32 * WAVES_N;
+    constexpr int RA = (BM * 8 + NTHREADS - 1) / NTHREADS, RB = (BN * 8 + NTHREADS - 1) / NTHREADS;
+
+    __shared__ __attribute__((aligned(16))) float As[2][BM][LD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN][LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int k_begin = blockIdx.z * a.k_chunk;
+    const int k_end = min(a.K, k_begin + a.k_chunk);
+    const int nkt = (k_end - k_begin + BK - 1) / BK;
+
+    float4 areg[RA], breg[RB];
+    auto load_tile = [&](int kt) {
+        const int k0 = k_begin + kt * BK;
+        #pragma unroll
+        for(int r = 0; r < RA; r++) {
+            const int v = tid + r * NTHREADS;
+            if((BM * 8) % NTHREADS == 0 || v < BM * 8)
+                areg[r] = load_row4(a.A, m0 + (v >> 3), a.M, a.lda, k0 + (v & 7) * 4, k_end, a.vec_ok);
+        }
+        #pragma unroll
+        for(int r = 0; r < RB; r++) {
+            const int v = tid + r * NTHREADS;
+            if((BN * 8) % NTHREADS == 0 || v < BN * 8)
+                breg[r] = load_row4(a.Bw, n0 + (v >> 3), a.N, a.ldb, k0 + (v & 7) * 4, k_end, a.vec_ok);
+        }
+    };
+    auto store_tile = [&](int buf) {
+        #pragma unroll
+        for(int r = 0; r < RA; r++) {
+            const int v = tid + r * NTHREADS;
+            if((BM * 8) % NTHREADS == 0 || v < BM * 8)
+                *reinterpret_cast<float4*>(&As[buf][v >> 3][(v & 7) * 4]) = areg[r];
+        }
+        #pragma unroll
+        for(int r = 0; r < RB; r++) {
+            const int v = tid + r * NTHREADS;
+            if((BN * 8) % NTHREADS == 0 || v < BN * 8)
+                *reinterpret_cast<float4*>(&Bs[buf][v >> 3][(v & 7) * 4]) = breg[r];
+        }
+    };
+
+    floatx16 acc[MT][NT];
+    #pragma unroll
+    for(int i = 0; i < MT; i++)
+        #pragma unroll
+        for(int j = 0; j < NT; j++)
+            #pragma unroll
+            for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    if(nkt > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+    for(int kt = 0; kt < nkt; kt++) {
+        const int buf = kt & 1;
+        if(kt + 1 < nkt) load_tile(kt + 1);
+        #pragma unroll
+        for(int q = 0; q < 4; q++) {
+            float4 av[MT], bv[NT];
+            #pragma unroll
+            for(int i = 0; i < MT; i++)
+                av[i] = *reinterpret_cast<const float4*>(&As[buf][(wm * MT + i) * 32 + l32][half * 16 + q * 4]);
+            #pragma unroll
+            for(int j = 0; j < NT; j++)
+                bv[j] = *reinterpret_cast<const float4*>(&Bs[buf][(wn * NT + j) * 32 + l32][half * 16 + q * 4]);
+            #pragma unroll
+            for(int i = 0; i < MT; i++)
+                #pragma unroll
+                for(int j = 0; j < NT; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].x, bv[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].y, bv[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].z, bv[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].w, bv[j].w, acc[i][j], 0, 0, 0);
+                }
+        }
+        if(kt + 1 < nkt) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    if(EPI == EPI_LSTM) {
+        // wave tile columns: tile j = gate j (i, f, g, o) of hidden unit hb*32 + lane%32
+        const int hb = blockIdx.x * WAVES_N + wn;
+        const int h = hb * 32 + l32;
+        if(h < a.H) {
+            #pragma unroll
+            for(int i = 0; i < MT; i++)
+                #pragma unroll
+                for(int r = 0; r < 16; r++) {
+                    const int m = m0 + (wm * MT + i) * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                    if(m >= a.M) continue;
+                    float pre[4];
+                    #pragma unroll
+                    for(int gate = 0; gate < 4; gate++) {
+                        const int n = hb * 128 + gate * 32 + l32;
+                        pre[gate] = nbl_act_apply(a.act, acc[i][gate % NT][r] + a.b[n]) + a.gx[(size_t)m * a.ldc + n];
+                    }
+                    const float gi = nbl_act_apply(NBL_ACT_LOGISTIC, pre[0]);
+                    const float gf = nbl_act_apply(NBL_ACT_LOGISTIC, pre[1]);
+                    const float gg = nbl_act_apply(NBL_ACT_TANH, pre[2]);
+                    const float go = nbl_act_apply(NBL_ACT_LOGISTIC, pre[3]);
+                    // c_t = c_{t-1}*f + i*g with each product rounded, as the reference's separate passes do
+                    const size_t e = (size_t)m * a.H + h;
+                    const float ig = __fmul_rn(gi, gg);
+                    const float cf = __fmul_rn(a.c[e], gf);
+                    const float ct = __fadd_rn(cf, ig);
+                    a.c[e] = ct;
+                    a.C[e] = __fmul_rn(nbl_act_apply(NBL_ACT_TANH, ct), go);
+                }
+        }
+        return;
+    }
+    float *__restrict__ Cout = a.C + (EPI == EPI_PARTIAL ? (size_t)blockIdx.z * a.M * a.ldc : 0);
+    #pragma unroll
+    for(int j = 0; j < NT; j++) {
+        const int n = n0 + (wn * NT + j) * 32 + l32;
+        if(n >= a.N) continue;
+        float gn = 1.0f, bn = 0.0f;
+        if(EPI == EPI_DIRECT) { bn = a.b[n]; if(a.has_scale) gn = a.g[n]; }
+        #pragma unroll
+        for(int i = 0; i < MT; i++)
+            #pragma unroll
+            for(int r = 0; r < 16; r++) {
+                const int m = m0 + (wm * MT + i) * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                if(m >= a.M) continue;
+                float v = acc[i][j][r];
+                if(EPI == EPI_DIRECT) {
+                    v = a.has_scale ? v * gn + bn : v + bn;
+                    v = nbl_act_apply(a.act, v);
+                }
+                Cout[(size_t)m * a.ldc + n] = v;
+            }
+    }
+}
+
+// y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n])
+__global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ y,
+                                     const float *__restrict__ g, const float *__restrict__ b,
+                                     int M, int N, int S, int act, int has_scale) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)M * N;
+    if(e >= total) return;
+    const int n = (int)(e % N);
+    float v = 0.0f;
+    for(int z = 0; z < S; z++) v += part[(size_t)z * total + e];
+    v = has_scale ? v * g[n] + b[n] : v + b[n];
+    y[e] = nbl_act_apply(act, v);
+}
+
+bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
+
+}  // namespace
+
+struct nbl_fc_plan {
+    unsigned I, O; int act; bool has_scale;
+    float *w_dev, *g_dev, *b_dev;
+    float *ws_dev; size_t ws_bytes;     // split-K partial sums, grown on demand
+};
+
+struct nbl_lstm_plan {
+    unsigned I, H, Hp;                  // Hp = H rounded up to 32
+    int sub_act;
+    float *ucat_dev;                    // [4*Hp][I]  input-side weights, interleaved gate order, BN scale folded in
+    float *wcat_dev;                    // [4*Hp][H]  recurrent-side weights, same order
+    float *bu_dev, *bw_dev;             // [4*Hp] biases (BN shift folded in); for a linear sub_act bw is folded into bu
+    float *gx_dev; float *h0_dev; float *c_dev; size_t gx_bytes, state_bytes;
+};
+
+namespace {
+
+int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, int N, int K,
+              const float *g, const float *b, int act, int has_scale, float **ws, size_t *ws_bytes) {
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.A = A; a.Bw = Bw; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K; a.ldc = N;
+    a.vec_ok = (K % 4 == 0) && aligned16(A) && aligned16(Bw);
+    a.g = g; a.b = b; a.act = act; a.has_scale = has_scale;
+    // tile: 32*MT rows of batch per wave row
+    const bool small_m = M <= 32;
+    const int BM = small_m ? 32 : (M <= 64 ? 64 : 128);
+    const int BN = 128;
+    const unsigned gm = nbl_div_up(M, BM), gn = nbl_div_up(N, BN);
+    // split K until the grid covers the chip about twice (weights are streamed once either way)
+    int S = 1;
+    const int ktiles = nbl_div_up(K, GEMM_BK);
+    if(ws) {
+        while(S < 16 && (size_t)gm * gn * S < 2u * ctx->num_cu && ktiles / (S * 2) >= 8) S *= 2;
+    }
+    a.k_chunk = nbl_div_up(ktiles, S) * GEMM_BK;
+    S = nbl_div_up(K, a.k_chunk);
+    dim3 grid(gn, gm, S), block(256);
+    if(S > 1) {
+        const size_t need = (size_t)S * M * N * sizeof(float);
+        if(*ws_bytes < need) {
+            int rc = nbl_free(ctx, *ws);
+            *ws = NULL; *ws_bytes = 0;
+            if(rc != NBL_OK) return rc;
+            if((rc = nbl_malloc(ctx, (void**)ws, need)) != NBL_OK) return rc;
+            *ws_bytes = need;
+        }
+        a.C = *ws;
+        if(BM == 32)       hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(split-k)");
+        const size_t total = (size_t)M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                           *ws, C, g, b, M, N, S, act, has_scale);
+        NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
+    } else {
+        if(BM == 32)       hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel");
+    }
+    return NBL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
+                const float *scale_host, const float *mean_host, const float *var_host,
+                unsigned I, unsigned O, int act, nbl_fc_plan **out) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, out != NULL, "nbl_fc_pack: out is NULL");
+    *out = NULL;
+    NBL_REQUIRE(ctx, weight_host && bias_host, "nbl_fc_pack: weight/bias is NULL");
+    NBL_REQUIRE(ctx, (scale_host != NULL) == (mean_host != NULL) && (scale_host != NULL) == (var_host != NULL),
+                "nbl_fc_pack: scale, mean and var must be given together");
+    NBL_REQUIRE(ctx, I && O, "nbl_fc_pack: zero dimension");
+    NBL_REQUIRE(ctx, nbl_act_valid(act), "nbl_fc_pack: undefined activation type %d", act);
+    if((size_t)I * O >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_pack: weight matrix too large");
+    nbl_fc_plan *p = new nbl_fc_plan();
+    p->I = I; p->O = O; p->act = act; p->has_scale = scale_host != NULL;
+    p->w_dev = p->g_dev = p->b_dev = p->ws_dev = NULL; p->ws_bytes = 0;
+    std::vector<float> g(O), b(O);
+    nbl_fold_batchnorm(bias_host, scale_host, mean_host, var_host, O, g.data(), b.data());
+    int rc;
+    if((rc = nbl_malloc(ctx, (void**)&p->w_dev, (size_t)I * O * sizeof(float))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->g_dev, O * sizeof(float))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->b_dev, O * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->w_dev, weight_host, (size_t)I * O * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->g_dev, g.data(), O * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->b_dev, b.data(), O * sizeof(float))) != NBL_OK) {
+        nbl_fc_plan_destroy(ctx, p);
+        return rc;
+    }
+    *out = p;
+    return NBL_OK;
+}
+
+int nbl_fc_plan_destroy(nbl_ctx *ctx, nbl_fc_plan *p) {
+    if(!ctx || !p) return NBL_EINVAL;
+    nbl_free(ctx, p->w_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev); nbl_free(ctx, p->ws_dev);
+    delete p;
+    return NBL_OK;
+}
+
+int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_fc_fwd: NULL argument");
+    if(B == 0) return NBL_OK;
+    if((size_t)B * plan->I >= (1ull << 31) || (size_t)B * plan->O >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd: tensors of 2^31 elements or more are not supported");
+    nbl_fc_plan *p = const_cast<nbl_fc_plan*>(plan);   // the split-K workspace is a cache
+    return launch_fc(ctx, x_dev, p->w_dev, y_dev, (int)B, (int)p->O, (int)p->I, p->g_dev, p->b_dev,
+                     p->act, p->has_scale ? 1 : 0, &p->ws_dev, &p->ws_bytes);
+}
+
+// ---- LSTM ----------------------------------------------------------------------------------------
+// file order of the eight sub-layers (lstm_layer.cc:194-206) and the gate each one feeds;
+// compute order of the gates inside a wave tile is i, f, g (cell candidate), o.
+int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *const *bias_host,
+                  const float *const *scale_host, const float *const *mean_host, const float *const *var_host,
+                  unsigned I, unsigned H, int sub_act, nbl_lstm_plan **out) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, out != NULL, "nbl_lstm_pack: out is NULL");
+    *out = NULL;
+    NBL_REQUIRE(ctx, weight_host && bias_host, "nbl_lstm_pack: weight/bias is NULL");
+    NBL_REQUIRE(ctx, (scale_host != NULL) == (mean_host != NULL) && (scale_host != NULL) == (var_host != NULL),
+                "nbl_lstm_pack: scale, mean and var must be given together");
+    NBL_REQUIRE(ctx, I && H, "nbl_lstm_pack: zero dimension");
+    NBL_REQUIRE(ctx, nbl_act_valid(sub_act), "nbl_lstm_pack: undefined activation type %d", sub_act);
+    for(int s = 0; s < 8; s++) {
+        NBL_REQUIRE(ctx, weight_host[s] && bias_host[s], "nbl_lstm_pack: sub-layer %d has a NULL array", s);
+        if(scale_host) NBL_REQUIRE(ctx, scale_host[s] && mean_host[s] && var_host[s],
+                                   "nbl_lstm_pack: sub-layer %d has a NULL batchnorm array", s);
+    }
+    // file slot of (side, gate): W side = 0..3, U side = 4..7; within a side the file order is i, f, o, c
+    static const int slot_of_gate[4] = { 0, 1, 3, 2 };   // gate i, f, g(c), o -> offset inside the side
+    nbl_lstm_plan *p = new nbl_lstm_plan();
+    memset(p, 0, sizeof(*p));
+    p->I = I; p->H = H; p->Hp = nbl_div_up(H, 32) * 32; p->sub_act = sub_act;
+    const unsigned Np = 4 * p->Hp;
+    std::vector<float> ucat((size_t)Np * I, 0.0f), wcat((size_t)Np * H, 0.0f), bu(Np, 0.0f), bw(Np, 0.0f);
+    std::vector<float> g(H), b(H);
+    for(int side = 0; side < 2; side++) {         // 0 = W (hidden), 1 = U (input)
+        const unsigned fan_in = side == 0 ? H : I;
+        std::vector<float> &cat = side == 0 ? wcat : ucat;
+        std::vector<float> &bias = side == 0 ? bw : bu;
+        for(int gate = 0; gate < 4; gate++) {
+            const int s = side * 4 + slot_of_gate[gate];
+            nbl_fold_batchnorm(bias_host[s], scale_host ? scale_host[s] : NULL, mean_host ? mean_host[s] : NULL,
+                               var_host ? var_host[s] : NULL, H, g.data(), b.data());
+            for(unsigned h = 0; h < H; h++) {
+                const size_t row = (size_t)(h / 32) * 128 + gate * 32 + (h % 32);
+                const float *src = weight_host[s] + (size_t)h * fan_in;
+                float *dst = cat.data() + row * fan_in;
+                // batchnorm scale folded into the row (1 when batch_normalize=0)
+                for(unsigned k = 0; k < fan_in; k++) dst[k] = scale_host ? (float)((double)src[k] * (double)g[h]) : src[k];
+                bias[row] = b[h];
+            }
+        }
+    }
+    // gate pre-activation = sub_act(U.x + bu) + sub_act(W.h + bw); for a linear sub_act the two biases merge
+    if(sub_act == NBL_ACT_LINEAR)
+        for(unsigned n = 0; n < Np; n++) { bu[n] = bu[n] + bw[n]; bw[n] = 0.0f; }
+    int rc;
+    if((rc = nbl_malloc(ctx, (void**)&p->ucat_dev, ucat.size() * sizeof(float))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->wcat_dev, wcat.size() * sizeof(float))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->bu_dev, Np * sizeof(float))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->bw_dev, Np * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->ucat_dev, ucat.data(), ucat.size() * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->wcat_dev, wcat.data(), wcat.size() * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->bu_dev, bu.data(), Np * sizeof(float))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->bw_dev, bw.data(), Np * sizeof(float))) != NBL_OK) {
+        nbl_lstm_plan_destroy(ctx, p);
+        return rc;
+    }
+    *out = p;
+    return NBL_OK;
+}
+
+int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *p) {
+    if(!ctx || !p) return NBL_EINVAL;
+    nbl_free(ctx, p->ucat_dev); nbl_free(ctx, p->wcat_dev); nbl_free(ctx, p->bu_dev); nbl_free(ctx, p->bw_dev);
+    nbl_free(ctx, p->gx_dev); nbl_free(ctx, p->h0_dev); nbl_free(ctx, p->c_dev);
+    delete p;
+    return NBL_OK;
+}
+
+int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_dev, float *cell_dev,
+                 unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_lstm_fwd: NULL argument");
+    if(T == 0 || B == 0) return NBL_OK;
+    const unsigned Np = 4 * p->Hp;
+    if((size_t)T * B * Np >= (1ull << 31) || (size_t)T * B * p->I >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_lstm_fwd: tensors of 2^31 elements or more are not supported");
+    int rc;
+    const size_t gx_need = (size_t)T * B * Np * sizeof(float), st_need = (size_t)B * p->H * sizeof(float);
+    if(p->gx_bytes < gx_need) {
+        if((rc = nbl_free(ctx, p->gx_dev)) != NBL_OK) return rc;
+        p->gx_dev = NULL; p->gx_bytes = 0;
+        if((rc = nbl_malloc(ctx, (void**)&p->gx_dev, gx_need)) != NBL_OK) return rc;
+        p->gx_bytes = gx_need;
+    }
+    if(p->state_bytes < st_need) {
+        if((rc = nbl_free(ctx, p->h0_dev)) != NBL_OK || (rc = nbl_free(ctx, p->c_dev)) != NBL_OK) return rc;
+        p->h0_dev = p->c_dev = NULL; p->state_bytes = 0;
+        if((rc = nbl_malloc(ctx, (void**)&p->h0_dev, st_need)) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->c_dev, st_need)) != NBL_OK) return rc;
+        p->state_bytes = st_need;
+    }
+    // zero initial hidden and cell state (first forward() of a fresh reference layer)
+    if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK)
+        return rc;
+    // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
+    if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
+                       p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
+    // recurrent half, one fused kernel per step; h_{t-1} is read straight from y[t-1]
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.Bw = p->wcat_dev; a.M = (int)B; a.N = (int)Np; a.K = (int)p->H; a.lda = (int)p->H; a.ldb = (int)p->H;
+    a.ldc = (int)Np; a.k_chunk = nbl_div_up(p->H, GEMM_BK) * GEMM_BK;
+    a.b = p->bw_dev; a.act = p->sub_act; a.c = p->c_dev; a.H = (int)p->H;
+    const size_t step = (size_t)B * p->H;
+    for(unsigned t = 0; t < T; t++) {
+        a.A = t == 0 ? p->h0_dev : y_dev + (size_t)(t - 1) * step;
+        a.C = y_dev + (size_t)t * step;
+        a.gx = p->gx_dev + (size_t)t * B * Np;
+        a.vec_ok = (p->H % 4 == 0) && aligned16(a.A) && aligned16(a.Bw);
+        dim3 grid(p->Hp / 32, nbl_div_up(B, 64), 1);
+        hipLaunchKernelGGL((gemm_nt_kernel<1, 4, 2, 1, EPI_LSTM>), grid, dim3(128), 0, ctx->stream, a);
+        NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(lstm)");
+    }
+    if(cell_dev)
+        NBL_HIP(ctx, hipMemcpyAsync(cell_dev, p->c_dev, st_need, hipMemcpyDeviceToDevice, ctx->stream));
+    return NBL_OK;
+}
+
+}  // extern "C"

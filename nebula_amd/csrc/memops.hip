@@ -1,0 +1,272 @@
+// The bandwidth-bound layers: pooling, shortcut, softmax, stand-alone activations, bias and
+// inference batchnorm.  Each kernel reads its input once and writes its output once; wherever the
+// layout allows, a lane moves 16 bytes per access.
+#include "nbl_internal.h"
+
+#include <cfloat>
+
+namespace {
+
+// ---- pooling -------------------------------------------------------------------------------------
+// One thread per output element, lanes along the output row (coalesced stores, overlapping window
+// reads served by L1/L2).  Tap order, sentinel and tie rule follow pooling_layer.cc:126-140:
+// rows then columns, taps outside the image read -1e8, strict '>' keeps the first maximum.
+template<bool IS_MAX, bool WRITE_INDEX>
+__global__ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
+                            unsigned total, int H, int W, int OH, int OW, int ksize, int stride, int pad) {
+    const unsigned o = blockIdx.x * blockDim.x + threadIdx.x;
+    if(o >= total) return;
+    const unsigned ow = o % OW, t = o / OW, oh = t % OH, plane = t / OH;   // plane = b*C + c
+    const int h0 = (int)oh * stride - pad, w0 = (int)ow * stride - pad;
+    const unsigned base = plane * (unsigned)(H * W);
+    float best = -1e8f, acc = 0.0f;
+    unsigned best_at = 0xffffffffu;
+    for(int i = 0; i < ksize; i++) {
+        const int ih = h0 + i;
+        const bool row_ok = (unsigned)ih < (unsigned)H;
+        for(int j = 0; j < ksize; j++) {
+            const int iw = w0 + j;
+            const bool ok = row_ok && (unsigned)iw < (unsigned)W;
+            const unsigned at = base + (unsigned)(ih * W + iw);
+            if(IS_MAX) {
+                const float v = ok ? x[at] : -1e8f;
+                if(v > best) { best = v; best_at = at; }
+            } else {
+                acc += ok ? x[at] : 0.0f;
+            }
+        }
+    }
+    if(IS_MAX) {
+        y[o] = best;
+        if(WRITE_INDEX) index[o] = best_at;
+    } else {
+        y[o] = acc / (float)(ksize * ksize);
+    }
+}
+
+// ---- shortcut ------------------------------------------------------------------------------------
+// y = act(prev + conn') where conn' is conn cropped to the common channel/height/width box and
+// sampled with stride = max(1, in_w/out_w), sample = max(1, out_w/in_w) (common/utils.cc:28-60).
+// Fast path: identical spatial size (stride = sample = 1, same H and W), 4 elements per lane.
+__global__ void shortcut_same_hw_kernel(const float4 *__restrict__ prev, const float4 *__restrict__ conn,
+                                        float4 *__restrict__ y, size_t total4, unsigned hw4,
+                                        unsigned in_c, unsigned out_c, int act) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= total4) return;
+    const size_t plane = e / hw4;                  // b*out_c + c
+    const unsigned c = (unsigned)(plane % out_c);
+    float4 v = prev[e];
+    if(c < in_c) {
+        const size_t b = plane / out_c;
+        const float4 r = conn[(b * in_c + c) * hw4 + (e - plane * hw4)];
+        v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+    }
+    v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
+    v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
+    y[e] = v;
+}
+
+__global__ void shortcut_general_kernel(const float *__restrict__ prev, const float *__restrict__ conn,
+                                        float *__restrict__ y, size_t total,
+                                        unsigned in_c, unsigned in_h, unsigned in_w,
+                                        unsigned out_c, unsigned out_h, unsigned out_w,
+                                        unsigned stride, unsigned sample, unsigned box_c, unsigned box_h,
+                                        unsigned box_w, int act) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= total) return;
+    const unsigned w = (unsigned)(e % out_w);
+    size_t t = e / out_w;
+    const unsigned h = (unsigned)(t % out_h); t /= out_h;
+    const unsigned c = (unsigned)(t % out_c);
+    const size_t b = t / out_c;
+    float v = prev[e];
+    // element (h, w) receives a residual when it sits on the sample grid inside the common box
+    if(c < box_c && h % sample == 0 && w % sample == 0 && h / sample < box_h && w / sample < box_w) {
+        const unsigned sh = h / sample * stride, sw = w / sample * stride;
+        v += conn[((b * in_c + c) * in_h + sh) * in_w + sw];
+    }
+    y[e] = nbl_act_apply(act, v);
+}
+
+// ---- softmax -------------------------------------------------------------------------------------
+// One block per row (softmax_layer.cc:85-106): row maximum, e = exp(x - max) evaluated in double and
+// rounded to float as the CPU code does, sum, divide.  The sum is a tree over floats where the CPU
+// code adds left to right; the difference is far inside the 1e-4 tolerance of this layer.
+__device__ __forceinline__ float wave_max(float v) {
+    for(int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    for(int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
+    __shared__ float red[4];
+    const float *in = x + (size_t)blockIdx.x * n;
+    float *out = y + (size_t)blockIdx.x * n;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    float m = -FLT_MAX;
+    for(unsigned j = tid; j < n; j += 256) m = fmaxf(m, in[j]);
+    m = wave_max(m);
+    if(lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float s = 0.0f;
+    for(unsigned j = tid; j < n; j += 256) {
+        const float e = (float)exp((double)(in[j] - m));
+        out[j] = e;
+        s += e;
+    }
+    s = wave_sum(s);
+    if(lane == 0) red[wave] = s;
+    __syncthreads();
+    s = (red[0] + red[1]) + (red[2] + red[3]);
+    for(unsigned j = tid; j < n; j += 256) out[j] = out[j] / s;
+}
+
+// ---- elementwise ---------------------------------------------------------------------------------
+__global__ void activation_kernel(float *__restrict__ x, size_t n, int act) {
+    const size_t i4 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if(i4 + 3 < n) {
+        float4 v = *reinterpret_cast<float4*>(x + i4);
+        v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
+        v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
+        *reinterpret_cast<float4*>(x + i4) = v;
+    } else {
+        for(size_t i = i4; i < n; i++) x[i] = nbl_act_apply(act, x[i]);
+    }
+}
+
+// y[b][c][s] = y * g[c] + b[c]   (bias only: g == NULL)
+__global__ void channel_affine_kernel(float *__restrict__ y, const float *__restrict__ g, const float *__restrict__ b,
+                                      size_t total, unsigned channel, unsigned size) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= total) return;
+    const unsigned c = (unsigned)((e / size) % channel);
+    y[e] = g ? y[e] * g[c] + b[c] : y[e] + b[c];
+}
+
+// y = (float)((double)(y - mean[c]) / (sqrt(var[c]) + 1e-5)) * scale[c], the two CPU passes of
+// common/batchnorm.cc:58-97 in one.
+__global__ void batchnorm_inference_kernel(float *__restrict__ y, const float *__restrict__ mean,
+                                           const float *__restrict__ var, const float *__restrict__ scale,
+                                           size_t total, unsigned channel, unsigned size) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= total) return;
+    const unsigned c = (unsigned)((e / size) % channel);
+    const float centered = __fsub_rn(y[e], mean[c]);
+    const float normed = (float)((double)centered / (sqrt((double)var[c]) + 0.00001));
+    y[e] = __fmul_rn(normed, scale[c]);
+}
+
+}  // namespace
+
+extern "C" {
+
+int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index_dev,
+                 unsigned B, unsigned C, unsigned H, unsigned W,
+                 unsigned ksize, unsigned stride, unsigned pad, int mode) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, x_dev && y_dev, "nbl_pool_fwd: NULL pointer");
+    NBL_REQUIRE(ctx, mode == NBL_POOL_MAX || mode == NBL_POOL_AVG, "nbl_pool_fwd: undefined pooling layer type %d", mode);
+    NBL_REQUIRE(ctx, C && H && W && ksize && stride, "nbl_pool_fwd: zero dimension");
+    if(B == 0) return NBL_OK;
+    const unsigned OH = nbl_pool_out_dim(H, stride, pad), OW = nbl_pool_out_dim(W, stride, pad);
+    const size_t total = (size_t)B * C * OH * OW, in_total = (size_t)B * C * H * W;
+    if(total == 0) return NBL_OK;
+    if(total >= (1ull << 31) || in_total >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_pool_fwd: tensors of 2^31 elements or more are not supported");
+    dim3 grid((unsigned)nbl_div_up_sz(total, 256)), block(256);
+    if(mode == NBL_POOL_MAX) {
+        if(index_dev)
+            hipLaunchKernelGGL((pool_kernel<true, true>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
+                               (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
+        else
+            hipLaunchKernelGGL((pool_kernel<true, false>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
+                               (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
+    } else {
+        hipLaunchKernelGGL((pool_kernel<false, false>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
+                           (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
+    }
+    NBL_LAUNCH_CHECK(ctx, "pool_kernel");
+    return NBL_OK;
+}
+
+int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev, float *y_dev, unsigned B,
+                     unsigned in_c, unsigned in_h, unsigned in_w,
+                     unsigned out_c, unsigned out_h, unsigned out_w, int act) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, prev_dev && conn_dev && y_dev, "nbl_shortcut_fwd: NULL pointer");
+    NBL_REQUIRE(ctx, in_c && in_h && in_w && out_c && out_h && out_w, "nbl_shortcut_fwd: zero dimension");
+    NBL_REQUIRE(ctx, nbl_act_valid(act), "nbl_shortcut_fwd: undefined activation type %d", act);
+    if(B == 0) return NBL_OK;
+    const size_t total = (size_t)B * out_c * out_h * out_w;
+    if(total >= (1ull << 40)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_shortcut_fwd: tensor too large");
+    const unsigned hw = out_h * out_w;
+    const bool same_hw = in_h == out_h && in_w == out_w;
+    const bool vec = same_hw && hw % 4 == 0 && (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0;
+    if(vec) {
+        const size_t total4 = total / 4;
+        hipLaunchKernelGGL(shortcut_same_hw_kernel, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0, ctx->stream,
+                           (const float4*)prev_dev, (const float4*)conn_dev, (float4*)y_dev, total4, hw / 4,
+                           in_c, out_c, act);
+    } else {
+        const unsigned stride = in_w / out_w > 1 ? in_w / out_w : 1;
+        const unsigned sample = out_w / in_w > 1 ? out_w / in_w : 1;
+        hipLaunchKernelGGL(shortcut_general_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                           prev_dev, conn_dev, y_dev, total, in_c, in_h, in_w, out_c, out_h, out_w, stride, sample,
+                           in_c < out_c ? in_c : out_c, in_h < out_h ? in_h : out_h, in_w < out_w ? in_w : out_w, act);
+    }
+    NBL_LAUNCH_CHECK(ctx, "shortcut kernel");
+    return NBL_OK;
+}
+
+int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned rows, unsigned n) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, x_dev && y_dev, "nbl_softmax_fwd: NULL pointer");
+    if(rows == 0 || n == 0) return NBL_OK;
+    hipLaunchKernelGGL(softmax_kernel, dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    NBL_LAUNCH_CHECK(ctx, "softmax_kernel");
+    return NBL_OK;
+}
+
+int nbl_activation_fwd(nbl_ctx *ctx, float *x_dev, size_t n, int act) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, nbl_act_valid(act), "nbl_activation_fwd: undefined activation type %d", act);
+    if(n == 0 || act == NBL_ACT_LINEAR) return NBL_OK;
+    NBL_REQUIRE(ctx, x_dev != NULL, "nbl_activation_fwd: NULL pointer");
+    NBL_REQUIRE(ctx, ((size_t)x_dev & 15) == 0, "nbl_activation_fwd: pointer must be 16-byte aligned");
+    const size_t threads = nbl_div_up_sz(n, 4);
+    hipLaunchKernelGGL(activation_kernel, dim3((unsigned)nbl_div_up_sz(threads, 256)), dim3(256), 0, ctx->stream,
+                       x_dev, n, act);
+    NBL_LAUNCH_CHECK(ctx, "activation_kernel");
+    return NBL_OK;
+}
+
+int nbl_forward_bias(nbl_ctx *ctx, float *y_dev, const float *bias_dev,
+                     unsigned channel, unsigned size, unsigned batch) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, y_dev && bias_dev, "nbl_forward_bias: NULL pointer");
+    const size_t total = (size_t)batch * channel * size;
+    if(total == 0) return NBL_OK;
+    hipLaunchKernelGGL(channel_affine_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                       y_dev, (const float*)NULL, bias_dev, total, channel, size);
+    NBL_LAUNCH_CHECK(ctx, "channel_affine_kernel");
+    return NBL_OK;
+}
+
+int nbl_batchnorm_inference(nbl_ctx *ctx, float *y_dev, const float *mean_dev, const float *var_dev,
+                            const float *scale_dev, unsigned channel, unsigned size, unsigned batch) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, y_dev && mean_dev && var_dev && scale_dev, "nbl_batchnorm_inference: NULL pointer");
+    const size_t total = (size_t)batch * channel * size;
+    if(total == 0) return NBL_OK;
+    hipLaunchKernelGGL(batchnorm_inference_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                       y_dev, mean_dev, var_dev, scale_dev, total, channel, size);
+    NBL_LAUNCH_CHECK(ctx, "batchnorm_inference_kernel");
+    return NBL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,88 @@
+// Internal declarations shared by the HIP translation units of libnebula_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "nebula_hip.h"
+
+struct nbl_ctx {
+    int device;
+    hipStream_t stream;
+    bool owns_stream;
+    hipEvent_t ev_start, ev_stop;
+    int num_cu;
+    char err[512];
+};
+
+// Records a formatted message on the context and returns `code`.
+int nbl_fail(nbl_ctx *ctx, int code, const char *fmt, ...);
+
+#define NBL_REQUIRE(ctx, cond, ...) \
+    do { if(!(cond)) return nbl_fail((ctx), NBL_EINVAL, __VA_ARGS__); } while(0)
+
+#define NBL_HIP(ctx, call) \
+    do { hipError_t e_ = (call); \
+         if(e_ != hipSuccess) return nbl_fail((ctx), e_ == hipErrorOutOfMemory ? NBL_ENOMEM : NBL_EHIP, \
+                                              "%s failed: %s", #call, hipGetErrorString(e_)); } while(0)
+
+// After a kernel launch: launch-configuration errors surface here.
+#define NBL_LAUNCH_CHECK(ctx, what) \
+    do { hipError_t e_ = hipGetLastError(); \
+         if(e_ != hipSuccess) return nbl_fail((ctx), NBL_EHIP, "launch of %s failed: %s", what, \
+                                              hipGetErrorString(e_)); } while(0)
+
+static inline unsigned nbl_div_up(unsigned a, unsigned b) { return (a + b - 1) / b; }
+static inline size_t nbl_div_up_sz(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// -------------------------------------------------------------------------------------------------
+// The thirteen activations of common/activations.cc:6-89, evaluated as the CPU file does: the
+// literals there are doubles, so anything that touches one is computed in double and rounded once
+// on the store.  relu / leaky / relie keep the `x > 0` predicate on the float value, which is what
+// makes their masks agree bit for bit.  elu, hardtan and lhtan are not the textbook functions
+// (elu squares positive inputs, the other two return 0/1 indicators); they are reproduced as written.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float nbl_act_apply(int act, float x) {
+    switch(act) {
+        case NBL_ACT_RELU:   return x > 0.0f ? x : 0.0f;
+        case NBL_ACT_LINEAR: return x;
+        case NBL_ACT_LEAKY:  return x > 0.0f ? x : (float)(0.1 * (double)x);
+        case NBL_ACT_RELIE:  return x > 0.0f ? x : (float)(0.01 * (double)x);
+        default: break;
+    }
+    const double d = (double)x;
+    switch(act) {
+        case NBL_ACT_ELU:      return x > 0.0f ? x * x : (float)(d * (exp(d) - 1.0));
+        case NBL_ACT_HARDTAN:  return (x < 1.0f && x > -1.0f) ? 1.0f : 0.0f;
+        case NBL_ACT_LHTAN:    return (x > 0.0f && x < 1.0f) ? 1.0f : 0.0f;
+        case NBL_ACT_LOGGY:    return (float)(2.0 / (1.0 + exp(0.0 - d)) - 1.0);
+        case NBL_ACT_LOGISTIC: return (float)(1.0 / (1.0 + exp(0.0 - d)));
+        case NBL_ACT_PLSE:
+            if(d < -4.0) return (float)(0.01 * (d + 4.0));
+            if(d > 4.0)  return (float)(0.01 * (d - 4.0) + 1.0);
+            return (float)(0.125 * d + 0.5);
+        case NBL_ACT_RAMP:     return x > 0.0f ? (float)(d * (d + 0.01)) : (float)(0.01 * d);
+        case NBL_ACT_STAIR: {
+            const int n = (int)x, half = (int)(d / 2.0);
+            return (n % 2) ? (x - (float)n) + (float)half : (float)half;
+        }
+        case NBL_ACT_TANH: {
+            const double e = exp(2.0 * d);
+            return (float)((e - 1.0) / (e + 1.0));
+        }
+        default: return x;
+    }
+}
+
+static inline bool nbl_act_valid(int act) { return act > NBL_ACT_UNDEFINED && act < NBL_ACT_COUNT; }
+
+// Inference batchnorm + bias as one multiply-add per channel, computed on the host in double:
+//   g = scale / (sqrt(var) + 1e-5)   (common/batchnorm.cc:70, eps outside the root)
+//   b = bias - mean * g
+// Without batchnorm g is 1 and b is the bias.
+void nbl_fold_batchnorm(const float *bias, const float *scale, const float *mean, const float *var,
+                        unsigned n, float *g_out, float *b_out);

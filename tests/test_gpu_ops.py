@@ -1,0 +1,298 @@
+"""Parity of every C-ABI entry point (include/nebula_hip.h) against the CPU oracle on the same
+seeded inputs.  Bars: bit-exact for the im2col gather, maxpool values + argmax, avgpool, shortcut,
+bias and the relu/leaky/relie activations; max|a-b| / max|ref| <= 1e-4 for conv / FC / LSTM /
+softmax / batchnorm and the exp-based activations."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as ob  # noqa: E402
+
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from nebula_amd import hip
+    c = hip.Ctx(0)
+    yield c
+    c.close()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32).ravel()
+
+
+def rel(a, b):
+    return float(np.abs(a.astype(np.float64) - b.astype(np.float64)).max() / max(float(np.abs(b).max()), 1e-30))
+
+
+def announce(*what):
+    print("CASE", *what, flush=True)
+
+
+IM2COL = [(3, 9, 9, 3, 1, 1), (2, 11, 7, 5, 2, 2), (3, 35, 35, 11, 4, 0), (4, 6, 8, 1, 1, 0), (2, 8, 8, 3, 2, 1),
+          (3, 14, 14, 7, 2, 3), (5, 10, 12, 3, 1, 0)]
+
+
+@pytest.mark.parametrize("shape", IM2COL)
+def test_im2col_gather_bit_exact(ctx, shape):
+    announce("im2col", shape)
+    c, h, w, k, s, p = shape
+    rng = np.random.default_rng(sum(shape))
+    im = rng.standard_normal((c, h, w)).astype(np.float32)
+    got = ctx.im2col(ctx.array(im), k, s, p).numpy()
+    want = ob.im2col(im, k, s, p)
+    assert got.shape == want.shape
+    np.testing.assert_array_equal(bits(got), bits(want))
+
+
+CONV = [
+    # B, C, H, W, F, k, s, p, bn, act
+    (2, 3, 12, 12, 5, 3, 1, 1, False, "linear"),
+    (3, 3, 35, 35, 16, 11, 4, 0, False, "relu"),          # AlexNet conv1 geometry
+    (2, 8, 14, 14, 40, 1, 1, 0, True, "leaky"),           # 1x1
+    (2, 16, 14, 14, 24, 3, 2, 1, True, "relu"),           # stride-2 3x3
+    (2, 3, 30, 30, 8, 7, 2, 3, True, "relu"),             # ResNet stem geometry
+    (1, 5, 9, 11, 130, 5, 1, 2, False, "logistic"),       # F > one m-tile, ragged K
+    (4, 32, 7, 7, 96, 3, 1, 1, True, "linear"),
+    (2, 4, 6, 6, 3, 2, 2, 1, False, "tanh"),
+]
+
+
+@pytest.mark.parametrize("case", CONV)
+def test_conv_matches_oracle(ctx, case):
+    from nebula_amd import hip
+    announce("conv", case)
+    B, Cc, H, W, F, k, s, p, bn, act = case
+    rng = np.random.default_rng(abs(hash(case[:8])) % (2 ** 31))
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    w = (rng.standard_normal((F, Cc, k, k)) * np.sqrt(2.0 / (Cc * k * k))).astype(np.float32)
+    bias = (rng.standard_normal(F) * 0.1).astype(np.float32)
+    bnp = None
+    if bn:
+        bnp = (rng.uniform(0.8, 1.2, F).astype(np.float32), (rng.standard_normal(F) * 0.1).astype(np.float32),
+               rng.uniform(0.5, 1.5, F).astype(np.float32))
+    want = ob.conv_forward(x, w, bias, bnp, s, p, act)
+    plan = ctx.conv_pack(w, bias, bnp, H=H, W=W, stride=s, pad=p, act=act)
+    dx = ctx.array(x)
+    for v in [-1] + list(range(hip.lib().nbl_conv2d_num_variants())):
+        announce("conv variant", v)
+        plan.set_variant(v)
+        got = plan(dx).numpy()
+        assert got.shape == want.shape
+        assert rel(got, want) <= TOL, (case, v, rel(got, want))
+
+
+def test_conv_relu_mask_matches_on_clear_margins(ctx):
+    # outputs further than the tolerance from zero must land on the same side of the ReLU
+    announce("conv relu mask")
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((2, 6, 16, 16)).astype(np.float32)
+    w = (rng.standard_normal((12, 6, 3, 3)) * 0.2).astype(np.float32)
+    b = (rng.standard_normal(12) * 0.1).astype(np.float32)
+    pre = ob.conv_forward(x, w, b, None, 1, 1, "linear")
+    want = ob.conv_forward(x, w, b, None, 1, 1, "relu")
+    got = ctx.conv_pack(w, b, None, H=16, W=16, stride=1, pad=1, act="relu")(ctx.array(x)).numpy()
+    clear = np.abs(pre) > 1e-4 * np.abs(pre).max()
+    np.testing.assert_array_equal((got > 0)[clear], (want > 0)[clear])
+
+
+@pytest.mark.parametrize("name", ob.ACT_NAMES[1:])
+def test_activation_kernels(ctx, name):
+    announce("activation", name)
+    rng = np.random.default_rng(ob.ACT[name])
+    x = np.concatenate([rng.standard_normal(70001) * 4, rng.uniform(-10, 10, 30000),
+                        np.arange(-9, 9.5, 0.5), [0.0, -0.0, 1e-30, -1e-30]]).astype(np.float32)
+    want = ob.activate(name, x)
+    got = ctx.activation(ctx.array(x), name).numpy()
+    if name in ("relu", "leaky", "relie", "linear", "hardtan", "lhtan", "plse", "ramp", "stair"):
+        np.testing.assert_array_equal(bits(got), bits(want))      # no transcendental involved
+    else:
+        ok = np.isfinite(want)
+        assert rel(got[ok], want[ok]) <= 1e-6
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    if name in ("relu", "leaky", "relie"):
+        np.testing.assert_array_equal(got > 0, x > 0)               # the mask itself
+
+
+def test_activation_rejects_undefined(ctx):
+    from nebula_amd import hip
+    d = ctx.array(np.zeros(8, np.float32))
+    for bad in (0, 14, -3):
+        rc = hip.lib().nbl_activation_fwd(ctx.h, d.ptr, 8, bad)
+        assert rc == -1
+        assert b"undefined activation" in hip.lib().nbl_last_error(ctx.h)
+
+
+POOL = [(2, 3, 12, 12, 3, 2, 1), (2, 2, 13, 11, 3, 2, 0), (1, 4, 8, 8, 2, 2, 0), (2, 5, 7, 7, 7, 7, 0),
+        (1, 2, 9, 9, 2, 1, 1), (1, 1, 6, 6, 5, 3, 2), (3, 16, 55, 55, 3, 2, 0), (2, 8, 112, 112, 3, 2, 0)]
+
+
+@pytest.mark.parametrize("geom", POOL)
+def test_maxpool_values_and_argmax_bit_exact(ctx, geom):
+    announce("maxpool", geom)
+    B, Cc, H, W, k, s, p = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    x[0, 0, :4, :4] = 0.25                      # ties: first maximum wins
+    x.ravel()[::17] = np.round(x.ravel()[::17])   # more ties
+    y, idx = ctx.pool(ctx.array(x), k, s, p, "max")
+    wy, widx = ob.maxpool_forward(x, k, s, p)
+    np.testing.assert_array_equal(bits(y.numpy()), bits(wy))
+    np.testing.assert_array_equal(idx.numpy(), widx)
+    y2, none = ctx.pool(ctx.array(x), k, s, p, "max", want_index=False)
+    assert none is None
+    np.testing.assert_array_equal(bits(y2.numpy()), bits(wy))
+
+
+def test_maxpool_sentinel(ctx):
+    announce("maxpool sentinel")
+    x = np.full((1, 1, 4, 4), -3e8, np.float32)
+    y, idx = ctx.pool(ctx.array(x), 2, 2, 0, "max")
+    wy, widx = ob.maxpool_forward(x, 2, 2, 0)
+    np.testing.assert_array_equal(bits(y.numpy()), bits(wy))
+    np.testing.assert_array_equal(idx.numpy(), widx)
+
+
+@pytest.mark.parametrize("geom", POOL)
+def test_avgpool_bit_exact(ctx, geom):
+    announce("avgpool", geom)
+    B, Cc, H, W, k, s, p = geom
+    rng = np.random.default_rng(sum(geom) + 1)
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    got = ctx.pool(ctx.array(x), k, s, p, "avg").numpy()
+    want = ob.avgpool_forward(x, k, s, p)
+    np.testing.assert_array_equal(bits(got), bits(want))
+
+
+SHORTCUT = [((2, 4, 9, 9), (2, 16, 9, 9)), ((2, 8, 10, 10), (2, 16, 5, 5)), ((1, 6, 19, 19), (1, 6, 10, 10)),
+            ((2, 8, 4, 4), (2, 4, 8, 8)), ((3, 5, 7, 7), (3, 5, 7, 7)), ((2, 16, 8, 8), (2, 16, 8, 8)),
+            ((2, 8, 12, 12), (2, 32, 12, 12)), ((2, 32, 12, 12), (2, 8, 12, 12))]
+
+
+@pytest.mark.parametrize("dims", SHORTCUT)
+@pytest.mark.parametrize("act", ["linear", "relu", "leaky"])
+def test_shortcut_bit_exact(ctx, dims, act):
+    announce("shortcut", dims, act)
+    conn_shape, out_shape = dims
+    rng = np.random.default_rng(sum(conn_shape) + sum(out_shape))
+    conn = rng.standard_normal(conn_shape).astype(np.float32)
+    prev = rng.standard_normal(out_shape).astype(np.float32)
+    want = ob.shortcut_forward(prev, conn, act)
+    got = ctx.shortcut(ctx.array(prev), ctx.array(conn), act).numpy()
+    np.testing.assert_array_equal(bits(got), bits(want))
+    # in place over prev
+    dprev = ctx.array(prev)
+    ctx.shortcut(dprev, ctx.array(conn), act, out=dprev)
+    np.testing.assert_array_equal(bits(dprev.numpy()), bits(want))
+
+
+FC = [(7, 60, 11, False, "linear"), (32, 512, 1000, False, "relu"), (64, 2048, 1000, False, "linear"),
+      (128, 1024, 256, True, "leaky"), (5, 33, 3, True, "logistic"), (33, 4096, 130, False, "relu"),
+      (1, 256, 64, False, "tanh")]
+
+
+@pytest.mark.parametrize("case", FC)
+def test_fc_matches_oracle(ctx, case):
+    announce("fc", case)
+    B, I, O, bn, act = case
+    rng = np.random.default_rng(B * 7 + I + O)
+    x = rng.standard_normal((B, I)).astype(np.float32)
+    w = (rng.standard_normal((O, I)) * np.sqrt(2.0 / I)).astype(np.float32)
+    b = (rng.standard_normal(O) * 0.1).astype(np.float32)
+    bnp = None
+    if bn:
+        bnp = (rng.uniform(0.8, 1.2, O).astype(np.float32), (rng.standard_normal(O) * 0.1).astype(np.float32),
+               rng.uniform(0.5, 1.5, O).astype(np.float32))
+    want = ob.connected_forward(x, w, b, bnp, act)
+    got = ctx.fc_pack(w, b, bnp, act)(ctx.array(x)).numpy()
+    assert rel(got, want) <= TOL, rel(got, want)
+
+
+def test_bias_and_batchnorm_primitives(ctx):
+    announce("bias/bn primitives")
+    rng = np.random.default_rng(31)
+    B, Cc, S = 3, 10, 77
+    y = rng.standard_normal((B, Cc, S)).astype(np.float32)
+    bias = rng.standard_normal(Cc).astype(np.float32)
+    mean = (rng.standard_normal(Cc) * 0.1).astype(np.float32)
+    var = rng.uniform(0.01, 2, Cc).astype(np.float32)
+    scale = rng.uniform(0.5, 1.5, Cc).astype(np.float32)
+    a = y.copy()
+    ob.oracle().orc_forward_bias(ob._fp(a), ob._fp(bias), Cc, S, B)
+    got = ctx.forward_bias(ctx.array(y), ctx.array(bias), Cc, S, B).numpy()
+    np.testing.assert_array_equal(bits(got), bits(a))
+    a = y.copy()
+    ob.oracle().orc_batchnorm_normalize(ob._fp(a), ob._fp(mean), ob._fp(var), Cc, S, B)
+    ob.oracle().orc_batchnorm_scale_down(ob._fp(a), ob._fp(scale), Cc, S, B)
+    got = ctx.batchnorm_inference(ctx.array(y), ctx.array(mean), ctx.array(var), ctx.array(scale), Cc, S, B).numpy()
+    assert rel(got, a) <= 1e-6
+
+
+@pytest.mark.parametrize("shape", [(6, 333), (64, 1000), (3, 10000), (1, 5), (128, 1000)])
+def test_softmax(ctx, shape):
+    announce("softmax", shape)
+    rng = np.random.default_rng(shape[1])
+    x = (rng.standard_normal(shape) * 5).astype(np.float32)
+    want = ob.softmax_forward(x)
+    got = ctx.softmax(ctx.array(x)).numpy()
+    assert rel(got, want) <= TOL
+    np.testing.assert_array_equal(got.argmax(1), want.argmax(1))
+    assert np.abs(got.sum(1) - 1).max() < 1e-5
+
+
+LSTM = [(3, 2, 5, 4, False, "linear"), (4, 3, 6, 5, True, "tanh"), (6, 8, 64, 96, False, "linear"),
+        (5, 64, 128, 128, True, "linear"), (3, 70, 40, 33, False, "linear")]
+
+
+@pytest.mark.parametrize("case", LSTM)
+def test_lstm_matches_oracle(ctx, case):
+    announce("lstm", case)
+    T, B, I, H, bn, act = case
+    rng = np.random.default_rng(T * 100 + B + I + H)
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    names = ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU")
+    wt = [(rng.uniform(-1, 1, (H, H if n[1] == "W" else I)) / np.sqrt(H)).astype(np.float32) for n in names]
+    bs = [(rng.uniform(-1, 1, H) / np.sqrt(H)).astype(np.float32) for n in names]
+    bnp = None
+    if bn:
+        bnp = ([rng.uniform(0.8, 1.2, H).astype(np.float32) for _ in names],
+               [(rng.standard_normal(H) * 0.1).astype(np.float32) for _ in names],
+               [rng.uniform(0.5, 1.5, H).astype(np.float32) for _ in names])
+    want, wcell = ob.lstm_forward(x, wt, bs, bnp, act, want_cell=True)
+    plan = ctx.lstm_pack(wt, bs, bnp, act)
+    cell = ctx.empty((B, H))
+    got = plan(ctx.array(x), cell=cell).numpy()
+    assert rel(got, want) <= TOL, rel(got, want)
+    assert rel(cell.numpy(), wcell[-1]) <= TOL
+    # a second call starts again from zero state
+    got2 = plan(ctx.array(x)).numpy()
+    np.testing.assert_array_equal(bits(got2), bits(got))
+
+
+def test_error_paths(ctx):
+    from nebula_amd import hip
+    import ctypes as C
+    l = hip.lib()
+    announce("error paths")
+    p = C.c_void_p()
+    w = np.zeros((2, 2, 3, 3), np.float32)
+    b = np.zeros(2, np.float32)
+    f = lambda a: a.ctypes.data_as(C.POINTER(C.c_float))
+    assert l.nbl_conv2d_pack(ctx.h, f(w), f(b), None, None, None, 2, 8, 8, 2, 3, 1, 1, 0, C.byref(p)) == -1   # act 0
+    assert l.nbl_conv2d_pack(ctx.h, f(w), f(b), None, None, None, 2, 8, 8, 2, 3, 0, 1, 11, C.byref(p)) == -1  # stride 0
+    assert l.nbl_conv2d_pack(ctx.h, None, f(b), None, None, None, 2, 8, 8, 2, 3, 1, 1, 11, C.byref(p)) == -1  # NULL w
+    assert l.nbl_conv2d_pack(ctx.h, f(w), f(b), f(b), None, None, 2, 8, 8, 2, 3, 1, 1, 11, C.byref(p)) == -1  # half a BN
+    assert l.nbl_conv2d_pack(ctx.h, f(w), f(b), None, None, None, 2, 1, 1, 2, 3, 1, 0, 11, C.byref(p)) == -1  # k > input
+    assert l.nbl_pool_fwd(ctx.h, None, None, None, 1, 1, 4, 4, 2, 2, 0, 0) == -1
+    d = ctx.empty((16,))
+    assert l.nbl_pool_fwd(ctx.h, d.ptr, d.ptr, None, 1, 1, 4, 4, 2, 2, 0, 7) == -1                             # mode
+    # zero batch is a no-op, not an error
+    plan = ctx.conv_pack(w, b, None, H=8, W=8, stride=1, pad=1, act="relu")
+    assert l.nbl_conv2d_fwd(ctx.h, plan.p, d.ptr, d.ptr, 0) == 0
+    assert l.nbl_ctx_create(99, C.byref(p)) != 0
+    assert b"device" in l.nbl_last_error(None)
