@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Forward-path benchmark.  One step = one forward pass of the workload over one synthetic batch that is
+already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|alexnet|vgg16|lstm|conv1]
+
+Default workload: ResNet-50 (the reference's own topology), fp32, batch 64 -- the configuration the
+headline metric is quoted on.  Besides the throughput the line carries
+  roofline:     the convolution kernel's algorithmic FLOP / its HIP-event time, against the fp32 MFMA peak
+  cpu_baseline: the reference's CPU algorithm (oracle port, OpenBLAS, all host cores) on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_weights(layout, rng, dist, lstm_hidden=1024):
+    """Synthetic weights in .wgh order from the network's own field table.  dist: 'he' (He-normal weights,
+    N(0,0.01) bias, or for normalised layers beta N(0,0.1), gamma U[0.8,1.2], mean N(0,0.1), var U[0.5,1.5])
+    or 'lstm' (everything U[-1/sqrt(H), 1/sqrt(H)])."""
+    normalised = {li for li, kind, _, _ in layout if kind == "scale"}
+    parts = []
+    for li, kind, count, fan_in in layout:
+        if dist == "lstm":
+            a = rng.uniform(-1, 1, count) / np.sqrt(lstm_hidden)
+        elif kind == "weight":
+            a = rng.standard_normal(count) * np.sqrt(2.0 / fan_in)
+        elif kind == "bias":
+            a = rng.standard_normal(count) * (0.1 if li in normalised else 0.01)
+        elif kind == "scale":
+            a = rng.uniform(0.8, 1.2, count)
+        elif kind == "mean":
+            a = rng.standard_normal(count) * 0.1
+        else:
+            a = rng.uniform(0.5, 1.5, count)
+        parts.append(a.astype(np.float32))
+    return np.concatenate(parts)
+
+
+def workload(name, batch):
+    from nebula_amd import zoo
+    table = {
+        "resnet50": (zoo.resnet50_cfg, 64, "normal", "he", "ResNet-50 (Nebula topology) fp32 forward, batch %d, 3x224x224 N(0,1)"),
+        "alexnet": (zoo.alexnet_cfg, 128, "uniform", "he", "AlexNet fp32 forward, batch %d, 3x227x227 U[0,1)"),
+        "vgg16": (zoo.vgg16_cfg, 32, "normal", "he", "VGG-16 fp32 forward, batch %d, 3x224x224 N(0,1)"),
+        "conv1": (zoo.conv1_pool_cfg, 32, "uniform", "he", "AlexNet conv1+ReLU+maxpool fp32, batch %d"),
+        "lstm": (zoo.lstm_cfg, 64, "normal", "lstm", "2-layer LSTM 1024/1024 T=64 + 10000-way projection, batch %d"),
+    }
+    fn, default_batch, xdist, wdist, text = table[name]
+    b = batch or default_batch
+    return fn(b), b, xdist, wdist, text % b
+
+
+def cpu_baseline(cfg_fn, specs_weights, xdist, sample_batch, is_lstm, rng):
+    """The reference's CPU algorithm (per-image im2col + sgemm, separate bias/BN/activation passes) through
+    the oracle port with OpenBLAS on all host cores, on a bounded sample of the same workload."""
+    from oracle import binding as ob
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count() or 1
+    cores = min(cores, len(os.sched_getaffinity(0)))
+    blas = ob.use_openblas(threads=cores)
+    if not blas:
+        ob.use_custom_gemm()
+        ob.set_threads(cores)
+    net = ob.OracleNet(cfg_fn(sample_batch))
+    net.load_weights(specs_weights)
+    if is_lstm:
+        T = net.net["time_steps"]
+        x = rng.standard_normal((T, sample_batch, net.net["input_size"])).astype(np.float32)
+    else:
+        shape = (sample_batch, net.net["channels"], net.net["height"], net.net["width"])
+        x = (rng.random(shape) if xdist == "uniform" else rng.standard_normal(shape)).astype(np.float32)
+    t0 = time.perf_counter()
+    outs = net.forward(x)
+    dt = time.perf_counter() - t0
+    ob.use_custom_gemm()
+    ob.set_threads(1)
+    return sample_batch / dt, cores, dt, ("OpenBLAS (scipy bundle)" if blas else "reference-style threaded GEMM"), x, outs
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1"])
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every layer is batch-parallel with no exchange; "
+                 "more GPUs would each take batch/N images). Re-run with --gpus 1.")
+
+    from nebula_amd.net import Network
+
+    cfg, batch, xdist, wdist, text = workload(args.workload, args.batch)
+    is_lstm = args.workload == "lstm"
+    rng = np.random.default_rng(20240611)
+    net = Network(cfg)
+    blob = make_weights(net.weight_layout(), rng, wdist)
+    log("workload:", text, "| weights: %.1f MB" % (blob.nbytes / 1e6))
+    with tempfile.NamedTemporaryFile("wb", suffix=".wgh", delete=False) as f:
+        f.write(blob.tobytes())
+        wpath = f.name
+    net.load_weights(wpath)
+    os.unlink(wpath)
+    n_in = net.batch_size * net.input_size
+    x = (rng.random(n_in, dtype=np.float32) if xdist == "uniform" else rng.standard_normal(n_in).astype(np.float32))
+    net.set_input(x)                     # resident in HBM before the timed region
+
+    for _ in range(args.warmup):
+        net.forward()
+    net.sync()
+    # timed region: K forward passes, synchronised on both sides; HIP events on the library's own stream
+    net.timer_start()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.forward()
+    ev_ms = net.timer_stop()
+    net.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    units = batch                         # images (or sequences) per step
+    value = units / (wall / args.steps)
+    log("timed %d steps: wall %.3f ms/step, events %.3f ms/step" % (args.steps, ms_per_step, ev_ms / args.steps))
+
+    # per-layer HIP-event timing over the same workload -> the dominant kernel's achieved rate
+    layer_ms = np.zeros(net.num_layers)
+    reps = max(3, min(10, args.steps))
+    for _ in range(reps):
+        layer_ms += np.array(net.forward_timed())
+    layer_ms /= reps
+    kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
+    flops = np.array([net.layer_flop(i) for i in range(net.num_layers)]) * (net.batch_size if not is_lstm else net.batch_size)
+    by_kind = {}
+    for k, ms in zip(kinds, layer_ms):
+        by_kind[k] = by_kind.get(k, 0.0) + ms
+    log("per-layer-kind ms:", {k: round(v, 3) for k, v in by_kind.items()})
+    if is_lstm:
+        # 2*B*(I+H)*4H per step per layer
+        lstm_flop = sum(2.0 * net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])
+                        * 4 * net.layer_info(i)["output_size"] for i, k in enumerate(kinds) if k == "lstm_layer")
+        dom_ms = by_kind.get("lstm_layer", 0.0)
+        n_launch = sum(k == "lstm_layer" for k in kinds)
+        achieved = lstm_flop / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
+        dom_name = "lstm (input GEMM + fused recurrent steps)"
+    else:
+        conv = [i for i, k in enumerate(kinds) if k == "convolutional_layer"]
+        dom_ms = float(layer_ms[conv].sum())
+        n_launch = len(conv)
+        achieved = float(flops[conv].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
+        dom_name = "conv_igemm_kernel"
+    roofline = {"bound": "mfma", "kernel": dom_name, "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4)}
+
+    result = {
+        "metric": "ResNet-50 fp32 fwd images/s (bs64, 1 GPU); conv GEMM % of fp32 MFMA peak" if args.workload == "resnet50"
+                  else "%s fp32 fwd %s/s (1 GPU)" % (args.workload, "sequences" if is_lstm else "images"),
+        "value": round(value, 2), "unit": "sequences/s" if is_lstm else "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded"},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu and args.cpu_sample != 0:
+        from nebula_amd import zoo
+        sample = args.cpu_sample if args.cpu_sample > 0 else {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4}[args.workload]
+        cfg_fn = (lambda b: zoo.WORKLOADS[args.workload](b))
+        ips, cores, dt, blas, xs, outs = cpu_baseline(cfg_fn, blob, xdist, sample, is_lstm, np.random.default_rng(7))
+        result["cpu_baseline"] = {"value": round(ips, 3), "unit": result["unit"], "cores": cores, "kind": "port",
+                                  "sample": "%d %s of the same workload, 1 timed forward (%.1f s), %s" % (
+                                      sample, "sequences" if is_lstm else "images", dt, blas)}
+        log("cpu baseline: %.2f %s on %d cores (%s)" % (ips, result["unit"], cores, blas))
+    net.close()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

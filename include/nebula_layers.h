@@ -1,0 +1,63 @@
+/*
+ * nebula_layers.h -- C entry points of libnebula_layers.so, the C++ layer framework
+ * (nebula_amd/host: network_t / layer_t classes with the reference's surface) driven from C,
+ * Python (ctypes) or any other FFI.  The classes themselves are the drop-in for
+ * models/layers/ and models/networks/network.{h,cc}; these functions stand in for the 38-line
+ * benchmark mains (benchmarks/<net>_<size>/main.cc:28-34: construct, init(), run()) and for the
+ * dataset drivers' load_data()/print_results() (models/networks/convolutional.cc:263-483,
+ * recurrent.cc:179-247), which feed tensors and read results.
+ *
+ * Every function returns 0 on success and a negative value on failure; nbl_net_last_error() then
+ * holds the message the reference would have printed before exit(1).
+ */
+#ifndef NEBULA_LAYERS_H
+#define NEBULA_LAYERS_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nbl_net nbl_net;
+
+/* cfg: path of a network.cfg (is_text = 0) or its contents (is_text = 1).  batch_override > 0 replaces
+ * the [net] section's batch=.  weight_path may be NULL or "" (load later with nbl_net_load_weights). */
+int nbl_net_create(const char *cfg, int is_text, unsigned batch_override, int device,
+                   const char *weight_path, nbl_net **out);
+int nbl_net_destroy(nbl_net *net);
+const char *nbl_net_last_error(void);
+/* network_t::init_weight(path): the headerless fp32 .wgh stream, layer by layer in cfg order. */
+int nbl_net_load_weights(nbl_net *net, const char *weight_path);
+int nbl_net_store_weights(nbl_net *net, const char *weight_path);
+/* The arrays of the .wgh stream in file order.  Each field is four unsigneds: layer index, kind
+ * (0 bias, 1 weight matrix, 2 batchnorm scale, 3 rolling mean, 4 rolling variance), element count, fan-in.
+ * Writes at most `capacity` fields to `fields` (may be NULL) and the total number to *num_fields. */
+int nbl_net_weight_layout(nbl_net *net, unsigned *fields, size_t capacity, size_t *num_fields);
+/* dims[0..5] = batch_size (rows, including time steps), time_step, input_size, input_h, input_w, input_c */
+int nbl_net_dims(nbl_net *net, unsigned *dims);
+int nbl_net_num_layers(nbl_net *net);
+/* info[0..7] = layer_type, activation_type, output_channel, output_height, output_width, output_size,
+ * input_size, padding */
+int nbl_net_layer_info(nbl_net *net, int layer, unsigned *info);
+/* 2*F*OH*OW*C*k*k for a convolutional layer, 2*I*O for a connected one, 0 otherwise (per input row) */
+int nbl_net_layer_flop(nbl_net *net, int layer, double *flop_per_row);
+/* host -> device input, [batch_size][input_size] floats */
+int nbl_net_set_input(nbl_net *net, const float *host, size_t count);
+/* network_t::forward(); asynchronous unless the net ends in a softmax (which copies to the host) */
+int nbl_net_forward(nbl_net *net);
+int nbl_net_sync(nbl_net *net);
+/* forward with a HIP event between layers: ms[i] = duration of layer i (num_layers entries) */
+int nbl_net_forward_timed(nbl_net *net, float *ms);
+/* device -> host copy of layer's output ([batch_size][output_size]) or maxpool argmax table */
+int nbl_net_layer_output(nbl_net *net, int layer, float *host, size_t count);
+int nbl_net_pool_index(nbl_net *net, int layer, unsigned *host, size_t count);
+/* the softmax layer skips its device->host copy when enabled = 0 (throughput measurement) */
+int nbl_net_softmax_copy(nbl_net *net, int enabled);
+/* the nbl_ctx* of the network (include/nebula_hip.h), e.g. for nbl_timer_start/stop */
+void *nbl_net_ctx(nbl_net *net);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -50,8 +50,9 @@ def build_layers(verbose=True):
     srcs = sorted(glob.glob(os.path.join(HOST, "*.cc")))
     if not srcs:
         return None
-    _run(["g++", "-O2", "-std=c++11", "-fPIC", "-shared", "-Wall", "-I", os.path.join(ROOT, "include"), "-I", HOST,
-          "-o", LAYERS_SO] + srcs + ["-L", LIBDIR, "-lnebula_hip", "-Wl,-rpath,$ORIGIN"])
+    _run(["g++", "-O2", "-std=c++11", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include",
+          "-I", os.path.join(ROOT, "include"), "-I", HOST,
+          "-o", LAYERS_SO] + srcs + ["-L", LIBDIR, "-lnebula_hip", "-L", "/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
     return LAYERS_SO
 
 

@@ -1,0 +1,190 @@
+#include "network.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <fstream>
+#include <sstream>
+#include <stdexcept>
+
+#include "config.h"
+#include "layers.h"
+
+namespace nebula {
+
+void nbl_check(nbl_ctx *ctx, int rc, const char *what) {
+    if(rc == NBL_OK) return;
+    std::ostringstream msg;
+    msg << "Error: " << what << " failed (" << rc << "): " << nbl_last_error(ctx);
+    throw std::runtime_error(msg.str());
+}
+
+network_t::network_t() :
+    run_type(UNDEFINED_RUN), num_threads(1),
+    learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
+    input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL),
+    input_layer(NULL), output_layer(NULL), num_layers(0) {}
+
+network_t::~network_t() {}
+
+void network_t::forward() {
+    for(unsigned i = 0; i < num_layers; i++) layers[i]->_forward_();
+}
+
+void network_t::backward() { throw std::runtime_error("Error: backward() is not part of the inference-only build"); }
+void network_t::update() { throw std::runtime_error("Error: update() is not part of the inference-only build"); }
+
+void network_t::init(const std::string m_run_type, const std::string m_network_config,
+                     const std::string m_data_config, const std::string m_input_weight) {
+    run_type = (run_type_t)lookup_type(run_type_str, NUM_RUN_TYPES, m_run_type);
+    if(run_type != TEST_RUN) throw std::runtime_error("Error: only the `test` (inference) run type is supported");
+    init_network(m_network_config);
+    init_data(m_data_config);
+    init_weight(m_input_weight);
+}
+
+void network_t::init_weight(const std::string m_input_weight) {
+    if(m_input_weight.size()) {
+        std::fstream weight_file(m_input_weight.c_str(), std::fstream::in | std::fstream::binary);
+        if(!weight_file.is_open()) throw std::runtime_error("Error: failed to open " + m_input_weight);
+        for(size_t i = 0; i < layers.size(); i++) layers[i]->init_weight(weight_file);
+    } else {
+        if(run_type == TEST_RUN)
+            throw std::runtime_error(std::string("Error: missing input weight for ") + run_type_str[run_type]);
+        for(size_t i = 0; i < layers.size(); i++) layers[i]->init_weight();
+    }
+}
+
+void network_t::store_weight(const std::string m_output_weight) {
+    if(!m_output_weight.size()) return;
+    std::fstream weight_file(m_output_weight.c_str(), std::fstream::out | std::fstream::binary);
+    if(!weight_file.is_open()) throw std::runtime_error("Error: failed to open " + m_output_weight);
+    for(size_t i = 0; i < layers.size(); i++) layers[i]->store_weight(weight_file);
+}
+
+// ---- inference_net_t -------------------------------------------------------------------------------
+inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
+    batch_override(m_batch_override), is_recurrent(false) {
+    run_type = TEST_RUN;
+    int rc = nbl_ctx_create(device, &ctx);
+    if(rc != NBL_OK) {
+        std::ostringstream msg;
+        msg << "Error: cannot create a device context (" << rc << "): " << nbl_last_error(NULL);
+        throw std::runtime_error(msg.str());
+    }
+}
+
+inference_net_t::~inference_net_t() {
+    for(size_t i = layers.size(); i > 0; i--) delete layers[i - 1];
+    for(size_t i = 0; i < events.size(); i++) (void)hipEventDestroy((hipEvent_t)events[i]);
+    if(input_data_dev) nbl_free(ctx, input_data_dev);
+    delete [] input_data;
+    if(ctx) nbl_ctx_destroy(ctx);
+}
+
+void inference_net_t::init_network(const std::string m_network_config) {
+    config_t config;
+    config.parse(m_network_config);
+    build(config);
+}
+
+void inference_net_t::init_from_stream(std::istream &cfg, const std::string m_input_weight) {
+    config_t config;
+    config.parse_stream(cfg);
+    build(config);
+    init_data("");
+    if(m_input_weight.size()) init_weight(m_input_weight);
+}
+
+// One pass over the sections, as the reference's two drivers do
+// (models/networks/convolutional.cc:52-122 for image nets, recurrent.cc:115-175 for recurrent nets;
+// a [net] section holding time_steps= selects the recurrent reading).
+void inference_net_t::build(config_t &config) {
+    if(config.sections.empty() || config.sections[0].name != "net")
+        throw std::runtime_error("Error: network config must start with a [net] section");
+    num_layers = (unsigned)config.sections.size() - 1;
+    layers.reserve(num_layers);
+    for(size_t i = 0; i < config.sections.size(); i++) {
+        section_config_t sc = config.sections[i];
+        if(sc.name == "net") {
+            sc.get_setting("num_threads", &num_threads);
+            sc.get_setting("learning_rate", &learning_rate);
+            sc.get_setting("momentum", &momentum);
+            sc.get_setting("decay", &decay);
+            sc.get_setting("height", &input_height);
+            sc.get_setting("width", &input_width);
+            sc.get_setting("channels", &input_channel);
+            sc.get_setting("batch", &batch_size);
+            if(batch_override) batch_size = batch_override;
+            input_size = input_height * input_width * input_channel;
+            if(sc.exists("time_steps")) {
+                is_recurrent = true;
+                sc.get_setting("input_size", &input_size);
+                sc.get_setting("time_steps", &time_step);
+                batch_size *= time_step;                 // rows = time steps x sequences, time-major
+            }
+            if(!batch_size || !input_size) throw std::runtime_error("Error: [net] gives an empty input");
+            continue;
+        }
+        layer_t *prev = layers.size() ? layers.back() : NULL;
+        layer_t *layer = NULL;
+        if(sc.name == "convolutional")   layer = new convolutional_layer_t(this, prev, CONVOLUTIONAL_LAYER);
+        else if(sc.name == "connected")  layer = new connected_layer_t(this, prev, CONNECTED_LAYER);
+        else if(sc.name == "dropout")    layer = new dropout_layer_t(this, prev, DROPOUT_LAYER);
+        else if(sc.name == "maxpool")    layer = new pooling_layer_t(this, prev, MAXPOOL_LAYER);
+        else if(sc.name == "avgpool")    layer = new pooling_layer_t(this, prev, AVGPOOL_LAYER);
+        else if(sc.name == "shortcut")   layer = new shortcut_layer_t(this, prev, SHORTCUT_LAYER);
+        else if(sc.name == "softmax")  { layer = new softmax_layer_t(this, prev, SOFTMAX_LAYER); output_layer = layer; }
+        else if(sc.name == "cost")       layer = new cost_layer_t(this, prev, COST_LAYER);
+        else if(sc.name == "lstm")       layer = new lstm_layer_t(this, prev, LSTM_LAYER);
+        else throw std::runtime_error("Error: unknown layer type " + sc.name);
+        if(layers.empty()) input_layer = layer;
+        layers.push_back(layer);            // owned from here on, also if init() throws
+        layer->init(sc);
+    }
+    num_layers = (unsigned)layers.size();
+    if(!output_layer && !layers.empty()) output_layer = layers.back();
+}
+
+void inference_net_t::init_data(const std::string) {
+    if(input_data_dev) return;
+    const size_t count = (size_t)batch_size * input_size;
+    input_data = new float[count]();
+    nbl_check(ctx, nbl_malloc(ctx, (void**)&input_data_dev, count * sizeof(float)), "nbl_malloc(input)");
+    nbl_check(ctx, nbl_fill_zero(ctx, input_data_dev, count * sizeof(float)), "nbl_fill_zero(input)");
+    // the first layer captured the (then NULL) input pointer lazily through input_dev(), nothing to patch
+}
+
+void inference_net_t::set_input(const float *host, size_t count) {
+    if(count != (size_t)batch_size * input_size) throw std::runtime_error("Error: input tensor has the wrong size");
+    nbl_check(ctx, nbl_h2d(ctx, input_data_dev, host, count * sizeof(float)), "nbl_h2d(input)");
+}
+
+void inference_net_t::load_data(const unsigned) {}
+void inference_net_t::print_results() {}
+
+void inference_net_t::run(const std::string) {
+    forward();
+    nbl_check(ctx, nbl_sync(ctx), "nbl_sync");
+}
+
+void inference_net_t::forward_timed(std::vector<float> &ms) {
+    hipStream_t stream = (hipStream_t)nbl_ctx_stream(ctx);
+    while(events.size() < (size_t)num_layers + 1) {
+        hipEvent_t e;
+        if(hipEventCreate(&e) != hipSuccess) throw std::runtime_error("Error: hipEventCreate failed");
+        events.push_back((void*)e);
+    }
+    for(unsigned i = 0; i < num_layers; i++) {
+        if(hipEventRecord((hipEvent_t)events[i], stream) != hipSuccess) throw std::runtime_error("Error: hipEventRecord failed");
+        layers[i]->_forward_();
+    }
+    if(hipEventRecord((hipEvent_t)events[num_layers], stream) != hipSuccess) throw std::runtime_error("Error: hipEventRecord failed");
+    if(hipEventSynchronize((hipEvent_t)events[num_layers]) != hipSuccess) throw std::runtime_error("Error: hipEventSynchronize failed");
+    ms.assign(num_layers, 0.0f);
+    for(unsigned i = 0; i < num_layers; i++)
+        if(hipEventElapsedTime(&ms[i], (hipEvent_t)events[i], (hipEvent_t)events[i + 1]) != hipSuccess)
+            throw std::runtime_error("Error: hipEventElapsedTime failed");
+}
+
+}  // namespace nebula

@@ -1,0 +1,100 @@
+// network_t: the caller of the forward path (the reference's models/networks/network.h:19-96 surface,
+// inference half) and inference_net_t, a driver that builds either kind of shipped network
+// (image nets and recurrent nets) from a network.cfg and feeds it tensors instead of datasets.
+//
+// Where the reference prints to std::cerr and calls exit(1), this code throws std::runtime_error
+// with the same text; a command-line driver may turn that back into exit(1).
+#ifndef NEBULA_HOST_NETWORK_H
+#define NEBULA_HOST_NETWORK_H
+
+#include <istream>
+#include <string>
+#include <vector>
+
+#include "def.h"
+#include "nebula_hip.h"
+
+namespace nebula {
+
+class layer_t;
+
+class network_t {
+public:
+    network_t();
+    virtual ~network_t();
+
+    // Forward propagation: layers[i]->_forward_() in cfg order (models/networks/network.cc:57-63).
+    void forward();
+    // Training is outside this build.
+    void backward();
+    void update();
+    // run type, network.cfg, data.cfg (unused by inference_net_t), weight file
+    void init(const std::string m_run_type, const std::string m_network_config,
+              const std::string m_data_config, const std::string m_input_weight = "");
+    virtual void run(const std::string m_output_weight = "") = 0;
+
+    run_type_t run_type;
+    unsigned num_threads;               // kept for cfg compatibility; the GPU path does not use it
+
+    float learning_rate, momentum, decay, cost;   // parsed, unused at inference
+
+    unsigned input_height, input_width, input_channel, input_size;
+    unsigned batch_size;                // already multiplied by time_step for recurrent nets
+    unsigned time_step;
+
+    float *input_data;                  // host staging buffer [batch_size][input_size]
+    float *input_label;                 // unused at inference
+    float *input_data_dev;              // device input [batch_size][input_size]
+
+    nbl_ctx *ctx;                       // takes the place of cublas_handle / cudnn_handle
+
+    // Opens the headerless fp32 .wgh stream and lets every layer read its fields in cfg order
+    // (models/networks/network.cc:99-122).
+    void init_weight(const std::string m_input_weight);
+    void store_weight(const std::string m_output_weight);
+
+    std::vector<layer_t*> layers;
+    layer_t *input_layer, *output_layer;
+    unsigned num_layers;
+
+protected:
+    virtual void init_network(const std::string m_network_config) = 0;
+    virtual void init_data(const std::string m_data_config) = 0;
+    virtual void load_data(const unsigned m_batch_index) = 0;
+    virtual void print_results() = 0;
+};
+
+class inference_net_t : public network_t {
+public:
+    // device: HIP device ordinal.  batch_override > 0 replaces `batch=` of the [net] section.
+    explicit inference_net_t(int device = 0, unsigned batch_override = 0);
+    ~inference_net_t();
+
+    // Build from cfg text instead of a file.
+    void init_from_stream(std::istream &cfg, const std::string m_input_weight = "");
+    // Copy a host tensor [batch_size][input_size] to the device input.
+    void set_input(const float *host, size_t count);
+    void run(const std::string m_output_weight = "");
+    bool recurrent() const { return is_recurrent; }
+
+    // forward() with a HIP event between layers; ms[i] = time of layer i.
+    void forward_timed(std::vector<float> &ms);
+
+protected:
+    void init_network(const std::string m_network_config);
+    void init_data(const std::string m_data_config);
+    void load_data(const unsigned m_batch_index);
+    void print_results();
+
+private:
+    void build(class config_t &config);
+    unsigned batch_override;
+    bool is_recurrent;
+    std::vector<void*> events;
+};
+
+// Throws std::runtime_error(nbl_last_error) when an ABI call fails.
+void nbl_check(nbl_ctx *ctx, int rc, const char *what);
+
+}  // namespace nebula
+#endif

@@ -1,0 +1,81 @@
+"""network.cfg text for the networks the benchmarks are quoted on.
+
+The topologies follow the reference's shipped cfgs (benchmarks/{alexnet,vgg,resnet,lstm}_large/network.cfg):
+same layer sequence, filter counts, strides and paddings.  ResNet-50 is the reference's own variant:
+bottlenecks [3,4,6,3] with the stride on the 3x3, `[shortcut] hops=4` residuals WITHOUT projection
+convolutions, a 3x3/s2 maxpool with padding=0 and a 7x7/s7 average pool.
+"""
+
+
+def _net(batch, h, w, c):
+    return "[net]\nbatch=%d\nheight=%d\nwidth=%d\nchannels=%d\n" % (batch, h, w, c)
+
+
+def _conv(filters, size, stride, padding, activation, bn=False):
+    return "\n[convolutional]\n%sfilters=%d\nsize=%d\nstride=%d\npadding=%d\nactivation=%s\n" % (
+        "batch_normalize=1\n" if bn else "", filters, size, stride, padding, activation)
+
+
+def _pool(kind, size, stride, padding=None):
+    return "\n[%s]\nsize=%d\nstride=%d\n%s" % (kind, size, stride, "" if padding is None else "padding=%d\n" % padding)
+
+
+def _fc(output, activation):
+    return "\n[connected]\noutput=%d\nactivation=%s\n" % (output, activation)
+
+
+_TAIL = "\n[softmax]\ngroups=1\n\n[cost]\ntype=l2\n"
+
+
+def conv1_pool_cfg(batch=32):
+    """AlexNet conv1 + ReLU + 3x3/s2 maxpool."""
+    return _net(batch, 227, 227, 3) + _conv(96, 11, 4, 0, "relu") + _pool("maxpool", 3, 2, 0)
+
+
+def alexnet_cfg(batch=128):
+    s = _net(batch, 227, 227, 3)
+    s += _conv(96, 11, 4, 0, "relu") + _pool("maxpool", 3, 2, 0)
+    s += _conv(256, 5, 1, 2, "relu") + _pool("maxpool", 3, 2, 0)
+    s += _conv(384, 3, 1, 1, "relu") + _conv(384, 3, 1, 1, "relu") + _conv(256, 3, 1, 1, "relu")
+    s += _pool("maxpool", 3, 2, 0)
+    s += _fc(4096, "relu") + "\n[dropout]\nprobability=0.5\n" + _fc(4096, "relu") + "\n[dropout]\nprobability=0.5\n"
+    s += _fc(1000, "linear") + _TAIL
+    return s
+
+
+def vgg16_cfg(batch=32):
+    s = _net(batch, 224, 224, 3)
+    for filters, reps in ((64, 2), (128, 2), (256, 3), (512, 3), (512, 3)):
+        for _ in range(reps):
+            s += _conv(filters, 3, 1, 1, "relu")
+        s += _pool("maxpool", 2, 2)
+    s += _fc(4096, "relu") + "\n[dropout]\nprobability=0.5\n" + _fc(4096, "relu") + "\n[dropout]\nprobability=0.5\n"
+    s += _fc(1000, "linear") + _TAIL
+    return s
+
+
+def resnet50_cfg(batch=64, activation="relu"):
+    s = _net(batch, 224, 224, 3)
+    s += _conv(64, 7, 2, 3, activation, bn=True) + _pool("maxpool", 3, 2, 0)
+    for stage, (width, blocks) in enumerate(((64, 3), (128, 4), (256, 6), (512, 3))):
+        for block in range(blocks):
+            stride = 2 if (stage > 0 and block == 0) else 1
+            s += _conv(width, 1, 1, 0, activation, bn=True)
+            s += _conv(width, 3, stride, 1, activation, bn=True)
+            s += _conv(4 * width, 1, 1, 0, "linear", bn=True)
+            s += "\n[shortcut]\nhops=4\nactivation=%s\n" % activation
+    s += _pool("avgpool", 7, 7, 0) + _fc(1000, "linear") + _TAIL
+    return s
+
+
+def lstm_cfg(batch=64, time_steps=64, input_size=1024, hidden=1024, layers=2, classes=10000):
+    s = "[net]\nbatch=%d\ninput_size=%d\ntime_steps=%d\n" % (batch, input_size, time_steps)
+    for _ in range(layers):
+        s += "\n[lstm]\noutput=%d\nactivation=linear\n" % hidden
+    s += _fc(classes, "linear") + _TAIL
+    return s
+
+
+WORKLOADS = {
+    "conv1": conv1_pool_cfg, "alexnet": alexnet_cfg, "vgg16": vgg16_cfg, "resnet50": resnet50_cfg, "lstm": lstm_cfg,
+}

@@ -38,3 +38,21 @@ def test_no_device_is_reported_not_crashed():
     assert l.nbl_pool_out_dim(55, 2, 0) == 27 and l.nbl_pool_out_dim(112, 2, 0) == 56
     assert l.nbl_conv_out_dim(227, 11, 4, 0) == 55 and l.nbl_conv_out_dim(224, 7, 2, 3) == 112
     assert l.nbl_conv2d_num_variants() >= 1
+
+
+def test_layers_library_exports_and_reports_missing_device():
+    import subprocess, sys
+    from nebula_amd import net
+    text = open(os.path.join(ROOT, "include", "nebula_layers.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(nbl_net_[a-z0-9_]+)\s*\(", text)))
+    l = net.lib()
+    for n in names:
+        assert hasattr(l, n), "library does not export " + n
+    assert set(names) == set(net.SIGNATURES)
+    code = ("import sys; sys.path.insert(0, %r); from nebula_amd.net import Network, NetworkError\n"
+            "try:\n    Network('[net]\\nbatch=1\\nheight=4\\nwidth=4\\nchannels=1\\n[softmax]\\n'); print('created')\n"
+            "except NetworkError as e:\n    print('error:', e)\n") % ROOT
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.startswith("created") or "device context" in out.stdout

@@ -1,0 +1,180 @@
+"""Whole cfg-described networks through the C++ layer framework (libnebula_layers.so, which calls
+the C ABI) against the committed golden vectors of the reference and against the CPU oracle."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as ob  # noqa: E402
+
+TOL = 1e-4
+NETS = sorted(os.path.basename(p)[:-4] for p in glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))
+              if not p.endswith("activations.npz"))
+
+
+def rel(a, b):
+    return float(np.abs(a.astype(np.float64) - b.astype(np.float64)).max() / max(float(np.abs(b).max()), 1e-30))
+
+
+@pytest.mark.parametrize("name", NETS)
+def test_golden_network(golden_dir, name):
+    from nebula_amd.net import Network
+    print("CASE golden network", name, flush=True)
+    g = np.load(os.path.join(golden_dir, name + ".npz"))
+    with Network(str(g["cfg"])) as net:
+        assert net.batch_size == int(g["batch_size"]) and net.time_step == int(g["time_step"])
+        net.load_weight_blob(g["weights"])
+        net.set_input(g["input"])
+        net.forward()
+        for i in range(net.num_layers):
+            info = net.layer_info(i)
+            dims = g["dims_%02d" % i]
+            assert info["output_size"] == dims[3], (name, i)
+            assert info["layer_type"] == dims[4] and info["activation_type"] == dims[5], (name, i)
+            if info["kind"] in ("convolutional_layer", "maxpool_layer", "avgpool_layer", "shortcut_layer"):
+                assert (info["output_channel"], info["output_height"], info["output_width"]) == tuple(dims[:3])
+            if info["kind"] == "cost_layer":
+                continue
+            got, want = net.output(i), g["out_%02d" % i]
+            assert rel(got, want) <= TOL, (name, i, info["kind"], rel(got, want))
+        last = [i for i in range(net.num_layers) if net.layer_info(i)["kind"] != "cost_layer"][-1]
+        rows = net.batch_size
+        got, want = net.output(last).reshape(rows, -1), g["out_%02d" % last].reshape(rows, -1)
+        np.testing.assert_array_equal(got.argmax(1), want.argmax(1))
+
+
+def test_maxpool_index_through_layer(golden_dir):
+    # identical input to the pooling layer -> identical argmax table: feed the pool layer directly
+    from nebula_amd.net import Network
+    cfg = "[net]\nbatch=2\nheight=13\nwidth=11\nchannels=3\n[maxpool]\nsize=3\nstride=2\n"
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 3, 13, 11)).astype(np.float32)
+    with Network(cfg) as net:
+        net.set_input(x)
+        net.forward()
+        wy, widx = ob.maxpool_forward(x, 3, 2, 1)
+        np.testing.assert_array_equal(net.output(0).view(np.uint32), wy.ravel().view(np.uint32))
+        np.testing.assert_array_equal(net.pool_index(0), widx.ravel())
+
+
+def test_cfg_errors_are_reported():
+    from nebula_amd.net import Network, NetworkError
+    with pytest.raises(NetworkError, match="unknown layer type"):
+        Network("[net]\nbatch=1\nheight=4\nwidth=4\nchannels=1\n[bogus]\nx=1\n")
+    with pytest.raises(NetworkError, match="undefined activation type"):
+        Network("[net]\nbatch=1\nheight=4\nwidth=4\nchannels=1\n[convolutional]\nfilters=2\nsize=3\nactivation=swish\n")
+    with pytest.raises(NetworkError, match="invalid config"):
+        Network("[net]\nbatch=1\nheight\n")
+    with pytest.raises(NetworkError, match="failed to open"):
+        Network("/nonexistent/network.cfg", is_text=False)
+    with Network("[net]\nbatch=1\nheight=4\nwidth=4\nchannels=1\n[connected]\noutput=3\nactivation=linear\n") as net:
+        with pytest.raises(NetworkError, match="no weights"):
+            net.forward()
+        with pytest.raises(NetworkError, match="shorter"):
+            net.load_weight_blob(np.zeros(5, np.float32))
+
+
+def test_weights_round_trip(tmp_path, golden_dir):
+    from nebula_amd.net import Network
+    g = np.load(os.path.join(golden_dir, "convnet_mixed.npz"))
+    with Network(str(g["cfg"])) as net:
+        net.load_weight_blob(g["weights"])
+        out = str(tmp_path / "out.wgh")
+        assert __import__("nebula_amd.net", fromlist=["lib"]).lib().nbl_net_store_weights(net.h, out.encode()) == 0
+        np.testing.assert_array_equal(np.fromfile(out, np.float32), g["weights"])
+
+
+def _random_weights(specs, rng):
+    parts = []
+    for li, name, shape in ob.weight_layout(specs):
+        base = name.split(".")[-1]
+        if base == "weight":
+            a = rng.standard_normal(shape) * np.sqrt(2.0 / int(np.prod(shape[1:])))
+        elif base == "bias":
+            a = rng.standard_normal(shape) * 0.1
+        elif base == "scale":
+            a = rng.uniform(0.8, 1.2, shape)
+        elif base == "mean":
+            a = rng.standard_normal(shape) * 0.1
+        else:
+            a = rng.uniform(0.5, 1.5, shape)
+        parts.append(a.astype(np.float32).ravel())
+    return np.concatenate(parts)
+
+
+MINI_RESNET = """
+[net]
+batch=4
+height=32
+width=32
+channels=3
+[convolutional]
+batch_normalize=1
+filters=16
+size=7
+stride=2
+padding=3
+activation=relu
+[maxpool]
+size=3
+stride=2
+padding=0
+""" + "".join("""
+[convolutional]
+batch_normalize=1
+filters=%d
+size=1
+stride=1
+padding=0
+activation=relu
+[convolutional]
+batch_normalize=1
+filters=%d
+size=3
+stride=%d
+padding=1
+activation=relu
+[convolutional]
+batch_normalize=1
+filters=%d
+size=1
+stride=1
+padding=0
+activation=linear
+[shortcut]
+hops=4
+activation=relu
+""" % (c, c, s, 4 * c) for c, s in [(16, 1), (16, 1), (32, 2), (32, 1)]) + """
+[avgpool]
+size=4
+stride=4
+padding=0
+[connected]
+output=10
+activation=linear
+[softmax]
+"""
+
+
+def test_mini_resnet_against_oracle():
+    from nebula_amd.net import Network
+    print("CASE mini resnet", flush=True)
+    rng = np.random.default_rng(42)
+    onet = ob.OracleNet(MINI_RESNET)
+    blob = _random_weights(onet.specs, rng)
+    onet.load_weights(blob)
+    x = rng.standard_normal((4, 3, 32, 32)).astype(np.float32)
+    ob.use_custom_gemm()
+    want = onet.forward(x)
+    with Network(MINI_RESNET) as net:
+        net.load_weight_blob(blob)
+        net.set_input(x)
+        net.forward()
+        for i in range(net.num_layers):
+            got = net.output(i)
+            assert rel(got, want[i].ravel()) <= TOL, (i, net.layer_info(i)["kind"], rel(got, want[i].ravel()))
+        logits = net.output(net.num_layers - 2).reshape(4, -1)
+        np.testing.assert_array_equal(logits.argmax(1), want[-2].reshape(4, -1).argmax(1))
