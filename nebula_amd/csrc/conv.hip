@@ -18,6 +18,7 @@
 // register staging: the loads of tile t+1 are issued before the MFMAs of tile t.
 #include "nbl_internal.h"
 
+#include <cmath>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -32,7 +33,8 @@ struct ConvArgs {
     const float *x; const float *wp; const int2 *ktab; const float *g; const float *b; float *y;
     int H, W, F, OW, OHW, CHW, stride, pad;
     int N;        // B * OH * OW
-    int Kp, Mp;
+    int K, Kp, Mp;
+    unsigned x_bytes;
     int act, has_scale;
     int tiles_m, tiles_n;
 };
@@ -56,30 +58,56 @@ __device__ __forceinline__ PixelCoord conv_pixel(int n, int N, int OHW, int OW, 
     return p;
 }
 
-// One element of the patch matrix: the reference's padding rule (taps outside the image read 0).
-__device__ __forceinline__ float conv_gather(const float *__restrict__ x, const PixelCoord &p, int2 ke,
-                                             int H, int W) {
+// True when tap (i, j) of table entry ke falls inside the image for pixel p (the reference's padding
+// rule: taps outside read 0).
+__device__ __forceinline__ bool conv_tap_inside(const PixelCoord &p, int2 ke, int H, int W) {
     const int ih = p.ih0 + (ke.y >> 16), iw = p.iw0 + (ke.y & 0xffff);
-    const bool inside = (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
-    return inside ? x[p.xbase + ke.x] : 0.0f;
+    return (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
 }
 
-template<int MT, int NT, int WAVES_M, int WAVES_N>
+// One element of the patch matrix.
+__device__ __forceinline__ float conv_gather(const float *__restrict__ x, const PixelCoord &p, int2 ke,
+                                             int H, int W) {
+    return conv_tap_inside(p, ke, H, W) ? x[p.xbase + ke.x] : 0.0f;
+}
+
+// Input reads go through a raw buffer descriptor: an offset at or past the end of the tensor returns 0
+// in hardware, so "outside the image", "past the last pixel column" and "past the last patch row" all
+// become one out-of-range offset and the loads need neither a branch nor a select on their result
+// (either would have to wait for the load before the MFMAs of the current tile could start).
+constexpr unsigned OOB_OFFSET = 0x80000000u;     // tensors are limited to < 2^31 bytes
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float *p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+// How a block gathers its slice of the patch matrix.
+enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
+       GATHER_NOPAD = 1,    // padding = 0: every tap of a real pixel is inside the image
+       GATHER_1X1_VEC4 = 2  // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
+};
+
+template<int MT, int NT, int WAVES_M, int WAVES_N, int GATHER, bool FAST_ACT>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N)
 void conv_igemm_kernel(const ConvArgs a) {
     constexpr int BK = CONV_BK;
     constexpr int NTHREADS = 64 * WAVES_M * WAVES_N;
     constexpr int BM = MT * 32 * WAVES_M, BN = NT * 32 * WAVES_N;
     constexpr int LDA = BM + 32, LDB = BN + 32;        // rows k and k+1 land in different bank halves
-    static_assert(NTHREADS % BN == 0 || BN % NTHREADS == 0, "pixel columns must split evenly over threads");
-    constexpr int COLS_PER_THREAD = BN > NTHREADS ? BN / NTHREADS : 1;
-    constexpr int KSTEP = BN >= NTHREADS ? 1 : NTHREADS / BN;   // k rows covered per pass
-    constexpr int RB = BK / KSTEP;                              // passes over the k-tile
-    constexpr int A_VEC = BK * BM / 4;                          // float4s in a weight tile
+    constexpr bool VEC4 = GATHER == GATHER_1X1_VEC4;
+    constexpr int NCOLS = VEC4 ? BN / 4 : BN;          // column groups a k row is split into
+    static_assert(NTHREADS % NCOLS == 0, "pixel columns must split evenly over threads");
+    constexpr int KGROUPS = NTHREADS / NCOLS;          // thread groups along k
+    static_assert(BK % KGROUPS == 0, "k rows must split evenly over thread groups");
+    constexpr int RB = BK / KGROUPS;                   // k rows gathered per thread
+    constexpr int A_VEC = BK * BM / 4;                 // float4s in a weight tile
     constexpr int RA = (A_VEC + NTHREADS - 1) / NTHREADS;
+    static_assert(RA <= 2, "weight tile needs at most two float4 per thread");
 
-    __shared__ float As[2][BK][LDA];
-    __shared__ float Bs[2][BK][LDB];
+    __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
@@ -90,48 +118,92 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const float *__restrict__ x = a.x;
-    const int k_first = (BN >= NTHREADS) ? 0 : tid / BN;
-    PixelCoord px[COLS_PER_THREAD];
-    #pragma unroll
-    for(int c = 0; c < COLS_PER_THREAD; c++)
-        px[c] = conv_pixel(n0 + (tid % BN) + c * NTHREADS, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.x, a.x_bytes);
+    const int ncol = tid % NCOLS;
+    // Scalar modes: one pixel column per thread, RB consecutive k rows, and the k rows of a wave are
+    // uniform (NCOLS is a multiple of 64), so the table entries travel through scalar registers.
+    // VEC4 mode: four pixel columns per thread, k rows strided by KGROUPS, no table (offset = k * H*W).
+    const int kgroup = VEC4 ? tid / NCOLS : __builtin_amdgcn_readfirstlane(tid / NCOLS);
+    const int krow0 = VEC4 ? kgroup : kgroup * RB;
+    // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past the
+    // last pixel re-reads the last group (its results are never stored), a row past the last patch row
+    // re-reads the last row and is zeroed when the tile is written to LDS.
+    const int ncol_first = VEC4 ? min(n0 + ncol * 4, a.N - 4) : n0 + ncol;
+    const PixelCoord px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
+    // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
+    const unsigned xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
+    const float *__restrict__ xpix = a.x + (VEC4 ? px.xbase : 0);
 
-    float breg[COLS_PER_THREAD][RB];
-    float4 areg[RA];
+    // Two register stages: the loads of tile t+2 are issued while tile t is multiplied and tile t+1 is
+    // still in flight, so every global load has two k-tiles of MFMA time to arrive.
+    struct Stage {
+        float b[VEC4 ? 1 : RB];
+        float4 b4[VEC4 ? RB : 1];
+        float4 a0, a1;
+        unsigned kvalid;
+    };
+    Stage st0, st1;
+    int2 ke[VEC4 ? 1 : RB];  // table entries of the next tile to gather
 
-    auto load_tile = [&](int kt) {
-        const int kbase = kt * BK;
-        #pragma unroll
-        for(int r = 0; r < RB; r++) {
-            // uniform over the wave: the table entry comes through scalar registers
-            const int kk = __builtin_amdgcn_readfirstlane(kbase + k_first + r * KSTEP);
-            const int2 ke = a.ktab[kk];
+    auto load_ktab = [&](int kt) {
+        if(!VEC4) {
+            const int2 *__restrict__ tp = a.ktab + kt * BK + krow0;
             #pragma unroll
-            for(int c = 0; c < COLS_PER_THREAD; c++) breg[c][r] = conv_gather(x, px[c], ke, a.H, a.W);
-        }
-        #pragma unroll
-        for(int r = 0; r < RA; r++) {
-            const int v = tid + r * NTHREADS;
-            if(A_VEC % NTHREADS == 0 || v < A_VEC) {
-                const int row = v / (BM / 4), col4 = v % (BM / 4);
-                areg[r] = *reinterpret_cast<const float4*>(a.wp + (size_t)(kbase + row) * a.Mp + m0 + col4 * 4);
-            }
+            for(int r = 0; r < RB; r++) ke[r] = tp[r];
         }
     };
-    auto store_tile = [&](int buf) {
-        #pragma unroll
-        for(int r = 0; r < RB; r++)
+    // kt may run past the last tile (the pipeline tail): the weight tile index is clamped, the table has
+    // all-padding tiles behind the last one, and the VEC4 path clamps its row; such a tile is never used.
+    auto load_tile = [&](Stage &st, int kt, int nkt) {
+        if(VEC4) {
+            st.kvalid = 0;
             #pragma unroll
-            for(int c = 0; c < COLS_PER_THREAD; c++)
-                Bs[buf][k_first + r * KSTEP][(tid % BN) + c * NTHREADS] = breg[c][r];
-        #pragma unroll
-        for(int r = 0; r < RA; r++) {
-            const int v = tid + r * NTHREADS;
-            if(A_VEC % NTHREADS == 0 || v < A_VEC) {
-                const int row = v / (BM / 4), col4 = v % (BM / 4);
-                *reinterpret_cast<float4*>(&As[buf][row][col4 * 4]) = areg[r];
+            for(int r = 0; r < RB; r++) {
+                const int k = kt * BK + krow0 + r * KGROUPS;
+                st.kvalid |= (k < a.K ? 1u : 0u) << r;
+                // 1x1: input plane = output plane
+                st.b4[r] = *reinterpret_cast<const float4*>(xpix + (size_t)min(k, a.K - 1) * a.OHW);
             }
+        } else {
+            #pragma unroll
+            for(int r = 0; r < RB; r++) {
+                unsigned off = xoff + (unsigned)ke[r].x * 4u;     // stays out of range when xoff is (tables hold < 2^29)
+                if(GATHER == GATHER_PADDED) off = conv_tap_inside(px, ke[r], a.H, a.W) ? off : OOB_OFFSET;
+                else if(ke[r].y < 0) off = OOB_OFFSET;            // uniform: padding row of the table
+                st.b[r] = buf_load(xres, off);
+            }
+        }
+        const float *__restrict__ wtile = a.wp + (size_t)min(kt, nkt - 1) * BK * a.Mp + m0;
+        {
+            const int row = tid / (BM / 4), col4 = tid % (BM / 4);
+            if(A_VEC >= NTHREADS || tid < A_VEC)
+                st.a0 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
+        }
+        if(RA > 1) {
+            const int v = tid + NTHREADS;
+            const int row = v / (BM / 4), col4 = v % (BM / 4);
+            if(A_VEC >= 2 * NTHREADS || v < A_VEC)
+                st.a1 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
+        }
+    };
+    auto store_tile = [&](const Stage &st, int buf) {
+        if(VEC4) {
+            #pragma unroll
+            for(int r = 0; r < RB; r++)
+                *reinterpret_cast<float4*>(&Bs[buf][krow0 + r * KGROUPS][ncol * 4]) =
+                    ((st.kvalid >> r) & 1u) ? st.b4[r] : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            #pragma unroll
+            for(int r = 0; r < RB; r++) Bs[buf][krow0 + r][ncol] = st.b[r];
+        }
+        {
+            const int row = tid / (BM / 4), col4 = tid % (BM / 4);
+            if(A_VEC >= NTHREADS || tid < A_VEC) *reinterpret_cast<float4*>(&As[buf][row][col4 * 4]) = st.a0;
+        }
+        if(RA > 1) {
+            const int v = tid + NTHREADS;
+            const int row = v / (BM / 4), col4 = v % (BM / 4);
+            if(A_VEC >= 2 * NTHREADS || v < A_VEC) *reinterpret_cast<float4*>(&As[buf][row][col4 * 4]) = st.a1;
         }
     };
 
@@ -143,49 +215,135 @@ void conv_igemm_kernel(const ConvArgs a) {
             #pragma unroll
             for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const int nkt = a.Kp / BK;
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
-    for(int kt = 0; kt < nkt; kt++) {
-        const int buf = kt & 1;
-        if(kt + 1 < nkt) load_tile(kt + 1);
+    // Rows and columns are dealt to the MFMA tiles of a wave interleaved: tile i of the wave holds rows
+    // l*MT + i (l = 0..31) and tile j holds columns l*NT + j.  A lane therefore finds the MT (NT)
+    // operand values of one k in adjacent LDS words and fetches them with one wide read at a
+    // compile-time offset, and in the epilogue it owns NT adjacent pixels of each of its rows.
+    const float *a_lane = &As[0][half][wm * MT * 32 + l32 * MT];
+    const float *b_lane = &Bs[0][half][wn * NT * 32 + l32 * NT];
+    auto compute_tile = [&](int buf) {
+        const float *ap = a_lane + buf * (BK * LDA), *bp = b_lane + buf * (BK * LDB);
+        float av[2][MT], bv[2][NT];
+        #pragma unroll
+        for(int i = 0; i < MT; i++) av[0][i] = ap[i];
+        #pragma unroll
+        for(int j = 0; j < NT; j++) bv[0][j] = bp[j];
         #pragma unroll
         for(int ks = 0; ks < BK / 2; ks++) {
-            const int kk = 2 * ks + half;
-            float av[MT], bv[NT];
-            #pragma unroll
-            for(int i = 0; i < MT; i++) av[i] = As[buf][kk][(wm * MT + i) * 32 + l32];
-            #pragma unroll
-            for(int j = 0; j < NT; j++) bv[j] = Bs[buf][kk][(wn * NT + j) * 32 + l32];
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if(ks + 1 < BK / 2) {           // operands of the next k-step, in flight behind this step's MFMAs
+                #pragma unroll
+                for(int i = 0; i < MT; i++) av[nxt][i] = ap[(ks + 1) * 2 * LDA + i];
+                #pragma unroll
+                for(int j = 0; j < NT; j++) bv[nxt][j] = bp[(ks + 1) * 2 * LDB + j];
+            }
+            __builtin_amdgcn_sched_barrier(0);
             #pragma unroll
             for(int i = 0; i < MT; i++)
                 #pragma unroll
                 for(int j = 0; j < NT; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cur][i], bv[cur][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if(kt + 1 < nkt) store_tile(buf ^ 1);
+    };
+
+    const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
+    st0.a0 = st0.a1 = st1.a0 = st1.a1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    load_ktab(0);
+    load_tile(st0, 0, nkt);
+    load_ktab(1);
+    load_tile(st1, 1, nkt);
+    load_ktab(2);
+    store_tile(st0, 0);
+    __syncthreads();
+
+    for(int kt = 0; kt < nkt; kt += 2) {
+        // tile kt is in LDS buffer 0, tile kt+1 is in flight in stage 1
+#ifndef NBL_EXP_NO_GLOBAL
+        load_tile(st0, kt + 2, nkt);
+        load_ktab(kt + 3);
+#endif
+        compute_tile(0);
+#ifndef NBL_EXP_NO_LDSWRITE
+        store_tile(st1, 1);
+#endif
+#ifndef NBL_EXP_NO_BARRIER
         __syncthreads();
+#endif
+        // tile kt+1 is in LDS buffer 1, tile kt+2 is in flight in stage 0
+#ifndef NBL_EXP_NO_GLOBAL
+        load_tile(st1, kt + 3, nkt);
+        load_ktab(kt + 4);
+#endif
+        compute_tile(1);
+#ifndef NBL_EXP_NO_LDSWRITE
+        store_tile(st0, 0);
+#endif
+#ifndef NBL_EXP_NO_BARRIER
+        __syncthreads();
+#endif
     }
 
-    // Epilogue: y = act(acc * g[f] + b[f]).  Accumulator register r of a 32x32 tile holds row
-    // 8*(r/4) + 4*(lane/32) + r%4 and column lane%32.
+    // Epilogue: y = act(acc * g[f] + b[f]).  Accumulator register r of a 32x32 MFMA tile holds tile row
+    // 8*(r/4) + 4*(lane/32) + r%4 and tile column lane%32; with the interleaving above that is
+    // filter row*MT + i and pixel (lane%32)*NT + j of the wave's sub-tile.
+    const int nbase = n0 + wn * NT * 32 + l32 * NT;
+    if(nbase >= a.N) return;
+    const int b0 = nbase / a.OHW, pix0 = nbase - b0 * a.OHW;
+    // the NT pixels of this lane are contiguous in memory when they sit in one image; then (and when the
+    // address is 8-byte aligned) a pair is written as one 64-bit store
+    const bool pair_ok = NT == 2 && pix0 + 1 < a.OHW && ((pix0 | a.OHW) & 1) == 0;
+    // Per-filter constants first, all loads in flight together: for each group q of four accumulator
+    // registers the lane's filters f = fq + rr*MT + i (rr = r%4) are 4*MT consecutive entries of the
+    // (zero padded) g and b vectors.
+    float gq[4][4 * MT], bq[4][4 * MT];
     #pragma unroll
-    for(int j = 0; j < NT; j++) {
-        const int n = n0 + (wn * NT + j) * 32 + l32;
-        if(n >= a.N) continue;
-        const int b = n / a.OHW, pix = n - b * a.OHW;
-        float *__restrict__ yb = a.y + (size_t)b * a.F * a.OHW + pix;
+    for(int q = 0; q < 4; q++) {
+        const int fq = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT;
         #pragma unroll
-        for(int i = 0; i < MT; i++) {
+        for(int v = 0; v < MT; v++) {
+            const float4 bb = *reinterpret_cast<const float4*>(a.b + fq + 4 * v);
+            bq[q][4 * v] = bb.x; bq[q][4 * v + 1] = bb.y; bq[q][4 * v + 2] = bb.z; bq[q][4 * v + 3] = bb.w;
+            if(a.has_scale) {
+                const float4 gg = *reinterpret_cast<const float4*>(a.g + fq + 4 * v);
+                gq[q][4 * v] = gg.x; gq[q][4 * v + 1] = gg.y; gq[q][4 * v + 2] = gg.z; gq[q][4 * v + 3] = gg.w;
+            }
+        }
+    }
+    float *__restrict__ ybase = a.y + (size_t)b0 * a.F * a.OHW + pix0;
+    #pragma unroll
+    for(int i = 0; i < MT; i++) {
+        #pragma unroll
+        for(int r = 0; r < 16; r++) {
+            const int q = r >> 2, e = (r & 3) * MT + i;
+            const int f = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT + e;
+            if(f >= a.F) continue;
+            const float bf = bq[q][e], gf = a.has_scale ? gq[q][e] : 1.0f;
+            float v[NT];
             #pragma unroll
-            for(int r = 0; r < 16; r++) {
-                const int f = m0 + (wm * MT + i) * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-                if(f < a.F) {
-                    float v = acc[i][j][r];
-                    v = a.has_scale ? v * a.g[f] + a.b[f] : v + a.b[f];
-                    yb[(size_t)f * a.OHW] = nbl_act_apply(a.act, v);
+            for(int j = 0; j < NT; j++) {
+                float t = acc[i][j][r];
+                t = a.has_scale ? t * gf + bf : t + bf;
+                if(FAST_ACT) {
+                    // relu / linear / leaky / relie: no transcendental, same predicates as nbl_act_apply
+                    if(a.act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
+                    else if(a.act == NBL_ACT_LEAKY) t = t > 0.0f ? t : (float)(0.1 * (double)t);
+                    else if(a.act == NBL_ACT_RELIE) t = t > 0.0f ? t : (float)(0.01 * (double)t);
+                } else {
+                    t = nbl_act_apply(a.act, t);
+                }
+                v[j] = t;
+            }
+            if(pair_ok) {
+                *reinterpret_cast<float2*>(ybase + (size_t)f * a.OHW) = make_float2(v[0], v[NT - 1]);
+            } else {
+                #pragma unroll
+                for(int j = 0; j < NT; j++) {
+                    const int n = nbase + j;
+                    if(n < a.N) {
+                        const int b = n / a.OHW, pix = n - b * a.OHW;
+                        a.y[((size_t)b * a.F + f) * a.OHW + pix] = v[j];
+                    }
                 }
             }
         }
@@ -212,21 +370,30 @@ std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, uns
             tab[kk].y = (int)((i << 16) | j);
         } else {
             tab[kk].x = 0;
-            tab[kk].y = KTAB_PAD_TAP << 16;
+            tab[kk].y = (int)0x80000000u | (KTAB_PAD_TAP << 16);   // sign bit: padding row
         }
     }
     return tab;
 }
 
-struct Variant { int bm, bn, threads; void (*kernel)(const ConvArgs); const char *name; };
+typedef void (*ConvKernel)(const ConvArgs);
+// kernel[gather mode][any activation ? 1 : 0]
+struct Variant { int bm, bn, threads; ConvKernel kernel[3][2]; const char *name; };
+
+#define NBL_CONV_VARIANT(MT, NT, WM, WN, NAME) \
+    { MT * 32 * WM, NT * 32 * WN, 64 * WM * WN, \
+      { { conv_igemm_kernel<MT, NT, WM, WN, GATHER_PADDED, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_PADDED, false> }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, GATHER_NOPAD, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_NOPAD, false> }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, GATHER_1X1_VEC4, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_1X1_VEC4, false> } }, \
+      NAME }
 
 const Variant VARIANTS[] = {
-    { 128, 128, 256, conv_igemm_kernel<2, 2, 2, 2>, "128x128" },
-    {  64, 256, 256, conv_igemm_kernel<2, 2, 1, 4>, "64x256" },
-    {  96, 256, 256, conv_igemm_kernel<3, 2, 1, 4>, "96x256" },
-    {  64, 128, 256, conv_igemm_kernel<1, 2, 2, 2>, "64x128" },
-    {  64,  64, 256, conv_igemm_kernel<1, 1, 2, 2>, "64x64" },
-    { 128,  64, 256, conv_igemm_kernel<2, 1, 2, 2>, "128x64" },
+    NBL_CONV_VARIANT(2, 2, 2, 2, "128x128"),
+    NBL_CONV_VARIANT(2, 2, 1, 4, "64x256"),
+    NBL_CONV_VARIANT(3, 2, 1, 4, "96x256"),
+    NBL_CONV_VARIANT(1, 2, 2, 2, "64x128"),
+    NBL_CONV_VARIANT(1, 1, 2, 2, "64x64"),
+    NBL_CONV_VARIANT(2, 1, 2, 2, "128x64"),
 };
 constexpr int NUM_VARIANTS = sizeof(VARIANTS) / sizeof(VARIANTS[0]);
 
@@ -237,6 +404,8 @@ struct nbl_conv_plan {
     int act; bool has_scale;
     float *wp_dev; int2 *ktab_dev; float *g_dev; float *b_dev;
     int variant;   // < 0: chosen per call
+    unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
+    bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
 };
 
 namespace {
@@ -286,9 +455,9 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->OH = nbl_conv_out_dim(H, ksize, stride, pad);
     p->OW = nbl_conv_out_dim(W, ksize, stride, pad);
     p->K = C * ksize * ksize;
-    p->Kp = nbl_div_up(p->K, CONV_BK) * CONV_BK;
+    p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
-    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
+    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false; p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL;
 
     // [F][K] -> [Kp][Mp], zero padded
@@ -297,7 +466,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
         for(unsigned kk = 0; kk < p->K; kk++) wp[(size_t)kk * p->Mp + f] = weight_host[(size_t)f * p->K + kk];
     std::vector<float> g(p->Mp, 0.0f), b(p->Mp, 0.0f);
     nbl_fold_batchnorm(bias_host, scale_host, mean_host, var_host, F, g.data(), b.data());
-    std::vector<int2> tab = build_ktab(C, H, W, ksize, p->Kp);
+    std::vector<int2> tab = build_ktab(C, H, W, ksize, p->Kp + 4 * CONV_BK);   // + all-padding tiles read by the pipeline tail
 
     int rc;
     if((rc = nbl_malloc(ctx, (void**)&p->wp_dev, wp.size() * sizeof(float))) != NBL_OK ||
@@ -336,20 +505,15 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
     return NBL_OK;
 }
 
-int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B) {
-    if(!ctx) return NBL_EINVAL;
-    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_conv2d_fwd: NULL argument");
-    if(B == 0) return NBL_OK;
-    const size_t in_elems = (size_t)B * p->C * p->H * p->W, out_elems = (size_t)B * p->F * p->OH * p->OW;
+static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v) {
+    const size_t in_elems = (size_t)B * p->C * p->H * p->W;
     const size_t npix = (size_t)B * p->OH * p->OW;
-    if(in_elems >= (1ull << 31) || out_elems >= (1ull << 31) || npix >= (1ull << 31) - 512)
-        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: tensors of 2^31 elements or more are not supported");
-    const int v = p->variant >= 0 ? p->variant : choose_variant(p, (unsigned)npix, ctx->num_cu);
     const Variant &var = VARIANTS[v];
     ConvArgs a;
     a.x = x_dev; a.wp = p->wp_dev; a.ktab = p->ktab_dev; a.g = p->g_dev; a.b = p->b_dev; a.y = y_dev;
     a.H = p->H; a.W = p->W; a.F = p->F; a.OW = p->OW; a.OHW = p->OH * p->OW; a.CHW = p->C * p->H * p->W;
-    a.stride = p->stride; a.pad = p->pad; a.N = (int)npix; a.Kp = p->Kp; a.Mp = p->Mp;
+    a.stride = p->stride; a.pad = p->pad; a.N = (int)npix; a.K = p->K; a.Kp = p->Kp; a.Mp = p->Mp;
+    a.x_bytes = (unsigned)(in_elems * sizeof(float));
     a.act = p->act; a.has_scale = p->has_scale ? 1 : 0;
     a.tiles_m = nbl_div_up(p->F, var.bm);
     a.tiles_n = nbl_div_up((unsigned)npix, var.bn);
@@ -358,9 +522,63 @@ int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, flo
         return nbl_fail(ctx, NBL_EINVAL, "nbl_conv2d_fwd: internal: tile %s overruns the packed weights", var.name);
     const size_t blocks = (size_t)a.tiles_m * a.tiles_n;
     if(blocks >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
-    hipLaunchKernelGGL(var.kernel, dim3((unsigned)blocks), dim3(var.threads), 0, ctx->stream, a);
+    const bool fast_act = p->act == NBL_ACT_RELU || p->act == NBL_ACT_LINEAR || p->act == NBL_ACT_LEAKY ||
+                          p->act == NBL_ACT_RELIE;
+    int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
+    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
+       !p->force_scalar_gather)
+        gather = GATHER_1X1_VEC4;
+    hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)blocks), dim3(var.threads), 0,
+                       ctx->stream, a);
     NBL_LAUNCH_CHECK(ctx, "conv_igemm_kernel");
     return NBL_OK;
+}
+
+// Tile search on the device: every tile shape runs the real problem twice and the faster second run
+// wins.  Block-count quantisation against the number of resident blocks decides more than any static
+// rule predicts, so the shapes are measured once per (layer, batch) and the result is kept in the plan.
+static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B) {
+    hipEvent_t e0, e1;
+    NBL_HIP(ctx, hipEventCreate(&e0));
+    hipError_t err = hipEventCreate(&e1);
+    if(err != hipSuccess) { (void)hipEventDestroy(e0); return nbl_fail(ctx, NBL_EHIP, "hipEventCreate: %s", hipGetErrorString(err)); }
+    int best = choose_variant(p, B * p->OH * p->OW, ctx->num_cu), rc = NBL_OK;
+    float best_ms = 1e30f;
+    for(int v = 0; v < NUM_VARIANTS && rc == NBL_OK; v++) {
+        if(nbl_div_up(p->F, VARIANTS[v].bm) * VARIANTS[v].bm > p->Mp) continue;
+        float ms = 0.0f;
+        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v)) != NBL_OK) break;
+        if(hipEventRecord(e0, ctx->stream) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed"); break; }
+        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v)) != NBL_OK) break;
+        if(hipEventRecord(e1, ctx->stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+           hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "event timing failed"); break; }
+        if(ms < best_ms) { best_ms = ms; best = v; }
+    }
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    if(rc != NBL_OK) return rc;
+    p->tuned_batch = B; p->tuned_variant = best;
+    return NBL_OK;
+}
+
+int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_conv2d_fwd: NULL argument");
+    if(B == 0) return NBL_OK;
+    nbl_conv_plan *p = const_cast<nbl_conv_plan*>(plan);      // the tile-search result is a cache
+    const size_t in_elems = (size_t)B * p->C * p->H * p->W, out_elems = (size_t)B * p->F * p->OH * p->OW;
+    const size_t npix = (size_t)B * p->OH * p->OW;
+    if(in_elems >= (1ull << 29) || out_elems >= (1ull << 31) || npix >= (1ull << 31) - 512)
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: inputs of 2^29 elements (2 GiB) or more are not supported");
+    int v = p->variant;
+    if(v < 0) {
+        if(p->tuned_batch != B) {
+            // the search overwrites y with correct results several times; tiny problems are not worth it
+            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); }
+            else { int rc = conv_tune(ctx, p, x_dev, y_dev, B); if(rc != NBL_OK) return rc; }
+        }
+        v = p->tuned_variant;
+    }
+    return conv_launch(ctx, p, x_dev, y_dev, B, v);
 }
 
 int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigned W,
