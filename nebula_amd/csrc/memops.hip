@@ -11,9 +11,13 @@ namespace {
 // One thread per output element, lanes along the output row (coalesced stores, overlapping window
 // reads served by L1/L2).  Tap order, sentinel and tie rule follow pooling_layer.cc:126-140:
 // rows then columns, taps outside the image read -1e8, strict '>' keeps the first maximum.
-template<bool IS_MAX, bool WRITE_INDEX>
-__global__ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
-                            unsigned total, int H, int W, int OH, int OW, int ksize, int stride, int pad) {
+// KS > 0 fixes the window size at compile time: all KS*KS loads are issued before the first compare
+// (addresses of taps outside the image are clamped and their values replaced), which is what lets
+// the kernel run at memory speed instead of one load latency per tap.  KS = 0 is the general loop.
+template<bool IS_MAX, bool WRITE_INDEX, int KS>
+__global__ __launch_bounds__(256)
+void pool_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
+                 unsigned total, int H, int W, int OH, int OW, int ksize, int stride, int pad) {
     const unsigned o = blockIdx.x * blockDim.x + threadIdx.x;
     if(o >= total) return;
     const unsigned ow = o % OW, t = o / OW, oh = t % OH, plane = t / OH;   // plane = b*C + c
@@ -21,18 +25,41 @@ __global__ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, 
     const unsigned base = plane * (unsigned)(H * W);
     float best = -1e8f, acc = 0.0f;
     unsigned best_at = 0xffffffffu;
-    for(int i = 0; i < ksize; i++) {
-        const int ih = h0 + i;
-        const bool row_ok = (unsigned)ih < (unsigned)H;
-        for(int j = 0; j < ksize; j++) {
-            const int iw = w0 + j;
-            const bool ok = row_ok && (unsigned)iw < (unsigned)W;
-            const unsigned at = base + (unsigned)(ih * W + iw);
-            if(IS_MAX) {
-                const float v = ok ? x[at] : -1e8f;
-                if(v > best) { best = v; best_at = at; }
-            } else {
-                acc += ok ? x[at] : 0.0f;
+    if(KS > 0) {
+        float v[KS > 0 ? KS * KS : 1];
+        #pragma unroll
+        for(int i = 0; i < KS; i++)
+            #pragma unroll
+            for(int j = 0; j < KS; j++) {
+                const int ih = h0 + i, iw = w0 + j;
+                const bool ok = (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+                const float val = x[base + (ok ? (unsigned)(ih * W + iw) : 0u)];
+                v[i * KS + j] = ok ? val : (IS_MAX ? -1e8f : 0.0f);
+            }
+        #pragma unroll
+        for(int i = 0; i < KS; i++)
+            #pragma unroll
+            for(int j = 0; j < KS; j++) {
+                if(IS_MAX) {
+                    if(v[i * KS + j] > best) { best = v[i * KS + j]; best_at = base + (unsigned)((h0 + i) * W + (w0 + j)); }
+                } else {
+                    acc += v[i * KS + j];
+                }
+            }
+    } else {
+        for(int i = 0; i < ksize; i++) {
+            const int ih = h0 + i;
+            const bool row_ok = (unsigned)ih < (unsigned)H;
+            for(int j = 0; j < ksize; j++) {
+                const int iw = w0 + j;
+                const bool ok = row_ok && (unsigned)iw < (unsigned)W;
+                const unsigned at = base + (unsigned)(ih * W + iw);
+                if(IS_MAX) {
+                    const float val = ok ? x[at] : -1e8f;
+                    if(val > best) { best = val; best_at = at; }
+                } else {
+                    acc += ok ? x[at] : 0.0f;
+                }
             }
         }
     }
@@ -42,6 +69,58 @@ __global__ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, 
     } else {
         y[o] = acc / (float)(ksize * ksize);
     }
+}
+
+// Stride 2, no padding, image width a multiple of 4: a lane produces two adjacent outputs from one
+// 16-byte load per window row (plus one scalar for the fifth column of a 3-wide window), so the
+// lanes of a wave read whole rows contiguously.  Same scan order, sentinel and tie rule as above.
+template<bool IS_MAX, bool WRITE_INDEX, int KS>
+__global__ __launch_bounds__(256)
+void pool_pair_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
+                      unsigned total_pairs, int H, int W, int OH, int OW2) {
+    const unsigned o2 = blockIdx.x * blockDim.x + threadIdx.x;
+    if(o2 >= total_pairs) return;
+    const unsigned t2 = o2 % OW2, t = o2 / OW2, oh = t % OH, plane = t / OH;
+    const unsigned base = plane * (unsigned)(H * W);
+    const int h0 = (int)oh * 2, w0 = (int)t2 * 4;
+    float v[KS][5];
+    #pragma unroll
+    for(int i = 0; i < KS; i++) {
+        const int ih = h0 + i;
+        const bool row_ok = ih < H;
+        const unsigned roff = base + (unsigned)((row_ok ? ih : 0) * W + w0);
+        const float4 q = *reinterpret_cast<const float4*>(x + roff);
+        const float pad_v = IS_MAX ? -1e8f : 0.0f;
+        v[i][0] = row_ok ? q.x : pad_v; v[i][1] = row_ok ? q.y : pad_v;
+        v[i][2] = row_ok ? q.z : pad_v; v[i][3] = row_ok ? q.w : pad_v;
+        if(KS == 3) {
+            const bool ok = row_ok && w0 + 4 < W;
+            const float e = x[ok ? roff + 4 : base];
+            v[i][4] = ok ? e : pad_v;
+        }
+    }
+    float out[2]; unsigned at[2];
+    #pragma unroll
+    for(int p = 0; p < 2; p++) {
+        float best = -1e8f, acc = 0.0f;
+        unsigned best_at = 0xffffffffu;
+        #pragma unroll
+        for(int i = 0; i < KS; i++)
+            #pragma unroll
+            for(int j = 0; j < KS; j++) {
+                const float val = v[i][2 * p + j];
+                if(IS_MAX) {
+                    if(val > best) { best = val; best_at = base + (unsigned)((h0 + i) * W + w0 + 2 * p + j); }
+                } else {
+                    acc += val;
+                }
+            }
+        out[p] = IS_MAX ? best : acc / (float)(KS * KS);
+        at[p] = best_at;
+    }
+    const size_t o = (size_t)o2 * 2;
+    *reinterpret_cast<float2*>(y + o) = make_float2(out[0], out[1]);
+    if(IS_MAX && WRITE_INDEX) *reinterpret_cast<uint2*>(index + o) = make_uint2(at[0], at[1]);
 }
 
 // ---- shortcut ------------------------------------------------------------------------------------
@@ -60,6 +139,36 @@ __global__ void shortcut_same_hw_kernel(const float4 *__restrict__ prev, const f
         const size_t b = plane / out_c;
         const float4 r = conn[(b * in_c + c) * hw4 + (e - plane * hw4)];
         v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+    }
+    v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
+    v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
+    y[e] = v;
+}
+
+// Spatial sizes differ by an integer stride and the output is not up-sampled (sample = 1): four
+// adjacent outputs per lane; with stride 2 their residuals are the even elements of 32 contiguous bytes.
+template<bool STRIDE2>
+__global__ void shortcut_strided_kernel(const float4 *__restrict__ prev, const float *__restrict__ conn,
+                                        float4 *__restrict__ y, size_t total4,
+                                        unsigned in_c, unsigned in_h, unsigned in_w,
+                                        unsigned out_c, unsigned out_h, unsigned out_w4,
+                                        unsigned stride, unsigned box_c, unsigned box_h, int act) {
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= total4) return;
+    const unsigned w4 = (unsigned)(e % out_w4);
+    size_t t = e / out_w4;
+    const unsigned h = (unsigned)(t % out_h); t /= out_h;
+    const unsigned c = (unsigned)(t % out_c);
+    const size_t b = t / out_c;
+    float4 v = prev[e];
+    if(c < box_c && h < box_h) {
+        const float *row = conn + ((b * in_c + c) * in_h + (size_t)h * stride) * in_w + (size_t)w4 * 4 * stride;
+        if(STRIDE2) {
+            const float4 r0 = *reinterpret_cast<const float4*>(row), r1 = *reinterpret_cast<const float4*>(row + 4);
+            v.x += r0.x; v.y += r0.z; v.z += r1.x; v.w += r1.z;
+        } else {
+            v.x += row[0]; v.y += row[stride]; v.z += row[2 * stride]; v.w += row[3 * stride];
+        }
     }
     v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
     v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
@@ -178,18 +287,38 @@ int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index
     if(total == 0) return NBL_OK;
     if(total >= (1ull << 31) || in_total >= (1ull << 31))
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_pool_fwd: tensors of 2^31 elements or more are not supported");
-    dim3 grid((unsigned)nbl_div_up_sz(total, 256)), block(256);
-    if(mode == NBL_POOL_MAX) {
-        if(index_dev)
-            hipLaunchKernelGGL((pool_kernel<true, true>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
-                               (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
-        else
-            hipLaunchKernelGGL((pool_kernel<true, false>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
-                               (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
-    } else {
-        hipLaunchKernelGGL((pool_kernel<false, false>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev,
-                           (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad);
+    // two outputs per lane from 16-byte loads
+    if(stride == 2 && pad == 0 && (ksize == 2 || ksize == 3) && W % 4 == 0 && OW == W / 2 && OW % 2 == 0 &&
+       (((size_t)x_dev | (size_t)y_dev | (size_t)index_dev) & 15) == 0) {
+        const unsigned pairs = (unsigned)(total / 2);
+        dim3 pgrid(nbl_div_up(pairs, 256)), pblock(256);
+#define NBL_PAIR_LAUNCH(IS_MAX, WI, KS) \
+        hipLaunchKernelGGL((pool_pair_kernel<IS_MAX, WI, KS>), pgrid, pblock, 0, ctx->stream, x_dev, y_dev, index_dev, \
+                           pairs, (int)H, (int)W, (int)OH, (int)(OW / 2))
+        if(mode == NBL_POOL_MAX) {
+            if(index_dev) { if(ksize == 2) NBL_PAIR_LAUNCH(true, true, 2); else NBL_PAIR_LAUNCH(true, true, 3); }
+            else          { if(ksize == 2) NBL_PAIR_LAUNCH(true, false, 2); else NBL_PAIR_LAUNCH(true, false, 3); }
+        } else {
+            if(ksize == 2) NBL_PAIR_LAUNCH(false, false, 2); else NBL_PAIR_LAUNCH(false, false, 3);
+        }
+#undef NBL_PAIR_LAUNCH
+        NBL_LAUNCH_CHECK(ctx, "pool_pair_kernel");
+        return NBL_OK;
     }
+    dim3 grid((unsigned)nbl_div_up_sz(total, 256)), block(256);
+#define NBL_POOL_LAUNCH(IS_MAX, WI, KS) \
+    hipLaunchKernelGGL((pool_kernel<IS_MAX, WI, KS>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev, \
+                       (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad)
+#define NBL_POOL_BY_K(IS_MAX, WI) \
+    do { switch(ksize) { case 2: NBL_POOL_LAUNCH(IS_MAX, WI, 2); break; case 3: NBL_POOL_LAUNCH(IS_MAX, WI, 3); break; \
+                         case 7: NBL_POOL_LAUNCH(IS_MAX, WI, 7); break; default: NBL_POOL_LAUNCH(IS_MAX, WI, 0); } } while(0)
+    if(mode == NBL_POOL_MAX) {
+        if(index_dev) NBL_POOL_BY_K(true, true); else NBL_POOL_BY_K(true, false);
+    } else {
+        NBL_POOL_BY_K(false, false);
+    }
+#undef NBL_POOL_BY_K
+#undef NBL_POOL_LAUNCH
     NBL_LAUNCH_CHECK(ctx, "pool_kernel");
     return NBL_OK;
 }
@@ -206,15 +335,36 @@ int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev,
     if(total >= (1ull << 40)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_shortcut_fwd: tensor too large");
     const unsigned hw = out_h * out_w;
     const bool same_hw = in_h == out_h && in_w == out_w;
-    const bool vec = same_hw && hw % 4 == 0 && (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0;
+    bool vec = same_hw && hw % 4 == 0 && (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0;
+    unsigned hw4 = hw / 4, vin_c = in_c, vout_c = out_c;
+    if(!vec && same_hw && in_c == out_c && ((size_t)out_c * hw) % 4 == 0 &&
+       (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0) {
+        // identical shapes: element e of conn adds to element e of prev; treat each image as one plane
+        vec = true; hw4 = (unsigned)((size_t)out_c * hw / 4); vin_c = vout_c = 1;
+    }
+    const unsigned stride = in_w / out_w > 1 ? in_w / out_w : 1;
+    const unsigned sample = out_w / in_w > 1 ? out_w / in_w : 1;
+    const bool aligned = (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0;
+    // four outputs per lane need the whole output row inside the common box and 16-byte aligned rows
+    const bool strided_vec = !same_hw && sample == 1 && out_w <= in_w && out_w % 4 == 0 && aligned &&
+                             (stride != 2 || in_w % 4 == 0);
     if(vec) {
         const size_t total4 = total / 4;
         hipLaunchKernelGGL(shortcut_same_hw_kernel, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0, ctx->stream,
-                           (const float4*)prev_dev, (const float4*)conn_dev, (float4*)y_dev, total4, hw / 4,
-                           in_c, out_c, act);
+                           (const float4*)prev_dev, (const float4*)conn_dev, (float4*)y_dev, total4, hw4,
+                           vin_c, vout_c, act);
+    } else if(strided_vec) {
+        const size_t total4 = total / 4;
+        const unsigned box_c = in_c < out_c ? in_c : out_c, box_h = in_h < out_h ? in_h : out_h;
+        if(stride == 2)
+            hipLaunchKernelGGL(shortcut_strided_kernel<true>, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0,
+                               ctx->stream, (const float4*)prev_dev, conn_dev, (float4*)y_dev, total4, in_c, in_h, in_w,
+                               out_c, out_h, out_w / 4, stride, box_c, box_h, act);
+        else
+            hipLaunchKernelGGL(shortcut_strided_kernel<false>, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0,
+                               ctx->stream, (const float4*)prev_dev, conn_dev, (float4*)y_dev, total4, in_c, in_h, in_w,
+                               out_c, out_h, out_w / 4, stride, box_c, box_h, act);
     } else {
-        const unsigned stride = in_w / out_w > 1 ? in_w / out_w : 1;
-        const unsigned sample = out_w / in_w > 1 ? out_w / in_w : 1;
         hipLaunchKernelGGL(shortcut_general_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
                            prev_dev, conn_dev, y_dev, total, in_c, in_h, in_w, out_c, out_h, out_w, stride, sample,
                            in_c < out_c ? in_c : out_c, in_h < out_h ? in_h : out_h, in_w < out_w ? in_w : out_w, act);

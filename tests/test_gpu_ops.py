@@ -129,7 +129,8 @@ def test_activation_rejects_undefined(ctx):
 
 
 POOL = [(2, 3, 12, 12, 3, 2, 1), (2, 2, 13, 11, 3, 2, 0), (1, 4, 8, 8, 2, 2, 0), (2, 5, 7, 7, 7, 7, 0),
-        (1, 2, 9, 9, 2, 1, 1), (1, 1, 6, 6, 5, 3, 2), (3, 16, 55, 55, 3, 2, 0), (2, 8, 112, 112, 3, 2, 0)]
+        (1, 2, 9, 9, 2, 1, 1), (1, 1, 6, 6, 5, 3, 2), (3, 16, 55, 55, 3, 2, 0), (2, 8, 112, 112, 3, 2, 0), (2, 4, 28, 28, 2, 2, 0),
+        (1, 3, 16, 12, 3, 2, 0), (2, 2, 14, 14, 7, 7, 0), (1, 2, 21, 21, 7, 2, 3)]
 
 
 @pytest.mark.parametrize("geom", POOL)
@@ -171,7 +172,8 @@ def test_avgpool_bit_exact(ctx, geom):
 
 SHORTCUT = [((2, 4, 9, 9), (2, 16, 9, 9)), ((2, 8, 10, 10), (2, 16, 5, 5)), ((1, 6, 19, 19), (1, 6, 10, 10)),
             ((2, 8, 4, 4), (2, 4, 8, 8)), ((3, 5, 7, 7), (3, 5, 7, 7)), ((2, 16, 8, 8), (2, 16, 8, 8)),
-            ((2, 8, 12, 12), (2, 32, 12, 12)), ((2, 32, 12, 12), (2, 8, 12, 12))]
+            ((2, 8, 12, 12), (2, 32, 12, 12)), ((2, 32, 12, 12), (2, 8, 12, 12)), ((2, 8, 7, 7), (2, 8, 7, 7)),
+            ((2, 8, 16, 16), (2, 24, 8, 8)), ((2, 6, 24, 24), (2, 6, 8, 8)), ((2, 4, 12, 12), (2, 8, 4, 4))]
 
 
 @pytest.mark.parametrize("dims", SHORTCUT)
