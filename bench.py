@@ -59,7 +59,8 @@ def workload(name, batch):
         "alexnet": (zoo.alexnet_cfg, 128, "uniform", "he", "AlexNet fp32 forward, batch %d, 3x227x227 U[0,1)"),
         "vgg16": (zoo.vgg16_cfg, 32, "normal", "he", "VGG-16 fp32 forward, batch %d, 3x224x224 N(0,1)"),
         "conv1": (zoo.conv1_pool_cfg, 32, "uniform", "he", "AlexNet conv1+ReLU+maxpool fp32, batch %d"),
-        "lstm": (zoo.lstm_cfg, 64, "normal", "lstm", "2-layer LSTM 1024/1024 T=64 + 10000-way projection, batch %d"),
+        "lstm": (lambda b: zoo.lstm_cfg(b, last_step_only=True), 64, "normal", "lstm",
+                 "2-layer LSTM 1024/1024 T=64 + 10000-way projection and softmax on the last step, batch %d"),
     }
     fn, default_batch, xdist, wdist, text = table[name]
     b = batch or default_batch
@@ -182,7 +183,7 @@ def main():
     if not args.no_cpu and args.cpu_sample != 0:
         from nebula_amd import zoo
         sample = args.cpu_sample if args.cpu_sample > 0 else {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4}[args.workload]
-        cfg_fn = (lambda b: zoo.WORKLOADS[args.workload](b))
+        cfg_fn = (lambda b: workload(args.workload, b)[0])
         ips, cores, dt, blas, xs, outs = cpu_baseline(cfg_fn, blob, xdist, sample, is_lstm, np.random.default_rng(7))
         result["cpu_baseline"] = {"value": round(ips, 3), "unit": result["unit"], "cores": cores, "kind": "port",
                                   "sample": "%d %s of the same workload, 1 timed forward (%.1f s), %s" % (

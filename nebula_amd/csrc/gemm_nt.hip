@@ -217,6 +217,37 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__re
     y[e] = nbl_act_apply(act, v);
 }
 
+// LSTM cell for one time step from split-K partial sums of the recurrent GEMM:
+//   pre[gate] = sub_act(sum_z part[z][m][n] + bw[n]) + gx[m][n],  n = (h/32)*128 + gate*32 + h%32
+//   i, f, o = logistic(pre), g = tanh(pre);  c = c*f + i*g;  h_out = tanh(c)*o
+// (lstm_layer.cc:264-312: each product is rounded on its own, as the separate CPU passes do).
+__global__ void lstm_cell_kernel(const float *__restrict__ part, const float *__restrict__ gx,
+                                 const float *__restrict__ bw, float *__restrict__ c, float *__restrict__ h_out,
+                                 int M, int H, int Np, int S, int sub_act) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if(e >= M * H) return;
+    const int m = e / H, h = e - m * H;
+    const int nbase = (h >> 5) * 128 + (h & 31);
+    const size_t plane = (size_t)M * Np;
+    float pre[4];
+    #pragma unroll
+    for(int gate = 0; gate < 4; gate++) {
+        const size_t at = (size_t)m * Np + nbase + gate * 32;
+        float acc = 0.0f;
+        for(int z = 0; z < S; z++) acc += part[(size_t)z * plane + at];
+        pre[gate] = nbl_act_apply(sub_act, acc + bw[nbase + gate * 32]) + gx[at];
+    }
+    const float gi = nbl_act_apply(NBL_ACT_LOGISTIC, pre[0]);
+    const float gf = nbl_act_apply(NBL_ACT_LOGISTIC, pre[1]);
+    const float gg = nbl_act_apply(NBL_ACT_TANH, pre[2]);
+    const float go = nbl_act_apply(NBL_ACT_LOGISTIC, pre[3]);
+    const float ig = __fmul_rn(gi, gg);
+    const float cf = __fmul_rn(c[e], gf);
+    const float ct = __fadd_rn(cf, ig);
+    c[e] = ct;
+    h_out[e] = __fmul_rn(nbl_act_apply(NBL_ACT_TANH, ct), go);
+}
+
 bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
 
 }  // namespace
@@ -234,6 +265,7 @@ struct nbl_lstm_plan {
     float *wcat_dev;                    // [4*Hp][H]  recurrent-side weights, same order
     float *bu_dev, *bw_dev;             // [4*Hp] biases (BN shift folded in); for a linear sub_act bw is folded into bu
     float *gx_dev; float *h0_dev; float *c_dev; size_t gx_bytes, state_bytes;
+    float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
 };
 
 namespace {
@@ -406,7 +438,7 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
 int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->ucat_dev); nbl_free(ctx, p->wcat_dev); nbl_free(ctx, p->bu_dev); nbl_free(ctx, p->bw_dev);
-    nbl_free(ctx, p->gx_dev); nbl_free(ctx, p->h0_dev); nbl_free(ctx, p->c_dev);
+    nbl_free(ctx, p->gx_dev); nbl_free(ctx, p->h0_dev); nbl_free(ctx, p->c_dev); nbl_free(ctx, p->part_dev);
     delete p;
     return NBL_OK;
 }
@@ -440,21 +472,48 @@ int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_de
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
     if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
                        p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
-    // recurrent half, one fused kernel per step; h_{t-1} is read straight from y[t-1]
+    // Recurrent half.  One step is only [B x H].[H x 4H]: to put work on every CU the k range is split
+    // over blockIdx.z into partial sums (deterministic order) and a small cell kernel finishes the step.
+    // Narrow problems keep the single fused kernel.  h_{t-1} is read straight from y[t-1].
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.Bw = p->wcat_dev; a.M = (int)B; a.N = (int)Np; a.K = (int)p->H; a.lda = (int)p->H; a.ldb = (int)p->H;
-    a.ldc = (int)Np; a.k_chunk = nbl_div_up(p->H, GEMM_BK) * GEMM_BK;
+    a.ldc = (int)Np;
     a.b = p->bw_dev; a.act = p->sub_act; a.c = p->c_dev; a.H = (int)p->H;
     const size_t step = (size_t)B * p->H;
+    const int ktiles = nbl_div_up(p->H, GEMM_BK);
+    const unsigned gm = nbl_div_up(B, 64), gn = Np / 128;
+    int S = 1;
+    while(S < 16 && (size_t)gm * gn * S < (size_t)ctx->num_cu && ktiles / (S * 2) >= 2) S *= 2;
+    a.k_chunk = nbl_div_up(ktiles, S) * GEMM_BK;
+    S = nbl_div_up(p->H, a.k_chunk);
+    if(S > 1) {
+        const size_t need = (size_t)S * B * Np * sizeof(float);
+        if(p->part_bytes < need) {
+            if((rc = nbl_free(ctx, p->part_dev)) != NBL_OK) return rc;
+            p->part_dev = NULL; p->part_bytes = 0;
+            if((rc = nbl_malloc(ctx, (void**)&p->part_dev, need)) != NBL_OK) return rc;
+            p->part_bytes = need;
+        }
+    }
     for(unsigned t = 0; t < T; t++) {
         a.A = t == 0 ? p->h0_dev : y_dev + (size_t)(t - 1) * step;
-        a.C = y_dev + (size_t)t * step;
         a.gx = p->gx_dev + (size_t)t * B * Np;
         a.vec_ok = (p->H % 4 == 0) && aligned16(a.A) && aligned16(a.Bw);
-        dim3 grid(p->Hp / 32, nbl_div_up(B, 64), 1);
-        hipLaunchKernelGGL((gemm_nt_kernel<1, 4, 2, 1, EPI_LSTM>), grid, dim3(128), 0, ctx->stream, a);
-        NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(lstm)");
+        if(S > 1) {
+            a.C = p->part_dev;
+            hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), dim3(gn, gm, S), dim3(256), 0, ctx->stream, a);
+            NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(lstm split-k)");
+            hipLaunchKernelGGL(lstm_cell_kernel, dim3(nbl_div_up((unsigned)step, 256)), dim3(256), 0, ctx->stream,
+                               p->part_dev, a.gx, p->bw_dev, p->c_dev, y_dev + (size_t)t * step,
+                               (int)B, (int)p->H, (int)Np, S, p->sub_act);
+            NBL_LAUNCH_CHECK(ctx, "lstm_cell_kernel");
+        } else {
+            a.C = y_dev + (size_t)t * step;
+            dim3 grid(p->Hp / 32, nbl_div_up(B, 64), 1);
+            hipLaunchKernelGGL((gemm_nt_kernel<1, 4, 2, 1, EPI_LSTM>), grid, dim3(128), 0, ctx->stream, a);
+            NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(lstm)");
+        }
     }
     if(cell_dev)
         NBL_HIP(ctx, hipMemcpyAsync(cell_dev, p->c_dev, st_need, hipMemcpyDeviceToDevice, ctx->stream));

@@ -64,7 +64,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    batch_override(m_batch_override), is_recurrent(false) {
+    last_step_only(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false) {
     run_type = TEST_RUN;
     int rc = nbl_ctx_create(device, &ctx);
     if(rc != NBL_OK) {
@@ -121,6 +121,7 @@ void inference_net_t::build(config_t &config) {
                 is_recurrent = true;
                 sc.get_setting("input_size", &input_size);
                 sc.get_setting("time_steps", &time_step);
+                sc.get_setting("last_step_only", &last_step_only);
                 batch_size *= time_step;                 // rows = time steps x sequences, time-major
             }
             if(!batch_size || !input_size) throw std::runtime_error("Error: [net] gives an empty input");
@@ -144,6 +145,8 @@ void inference_net_t::build(config_t &config) {
     }
     num_layers = (unsigned)layers.size();
     if(!output_layer && !layers.empty()) output_layer = layers.back();
+    for(unsigned i = 0; i < num_layers; i++)
+        if(layers[i]->layer_type == LSTM_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
 }
 
 void inference_net_t::init_data(const std::string) {
@@ -168,6 +171,29 @@ void inference_net_t::run(const std::string) {
     nbl_check(ctx, nbl_sync(ctx), "nbl_sync");
 }
 
+// Layer i, with the rows narrowed to the final time step from the first layer after the last LSTM on
+// when last_step_only is set: that layer reads the last B rows of its producer, everything after it
+// works on B rows.  The pointer and the row count are restored right after the call.
+void inference_net_t::run_layer(unsigned i) {
+    const bool narrow = last_step_only && is_recurrent && time_step > 1 && first_after_lstm >= 0 &&
+                        (int)i >= first_after_lstm;
+    if(!narrow) { layers[i]->_forward_(); return; }
+    const unsigned rows = batch_size, seqs = batch_size / time_step;
+    layer_t *producer = layers[i]->prev_layer;
+    float *saved = producer ? producer->output_data_dev : NULL;
+    if((int)i == first_after_lstm && producer)
+        producer->output_data_dev += (size_t)(time_step - 1) * seqs * producer->output_size;
+    batch_size = seqs;
+    try { layers[i]->_forward_(); }
+    catch(...) { batch_size = rows; if(producer) producer->output_data_dev = saved; throw; }
+    batch_size = rows;
+    if(producer) producer->output_data_dev = saved;
+}
+
+void inference_net_t::forward() {
+    for(unsigned i = 0; i < num_layers; i++) run_layer(i);
+}
+
 void inference_net_t::forward_timed(std::vector<float> &ms) {
     hipStream_t stream = (hipStream_t)nbl_ctx_stream(ctx);
     while(events.size() < (size_t)num_layers + 1) {
@@ -177,7 +203,7 @@ void inference_net_t::forward_timed(std::vector<float> &ms) {
     }
     for(unsigned i = 0; i < num_layers; i++) {
         if(hipEventRecord((hipEvent_t)events[i], stream) != hipSuccess) throw std::runtime_error("Error: hipEventRecord failed");
-        layers[i]->_forward_();
+        run_layer(i);
     }
     if(hipEventRecord((hipEvent_t)events[num_layers], stream) != hipSuccess) throw std::runtime_error("Error: hipEventRecord failed");
     if(hipEventSynchronize((hipEvent_t)events[num_layers]) != hipSuccess) throw std::runtime_error("Error: hipEventSynchronize failed");

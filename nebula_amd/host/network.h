@@ -77,8 +77,14 @@ public:
     void run(const std::string m_output_weight = "");
     bool recurrent() const { return is_recurrent; }
 
+    // network_t::forward(), plus the `last_step_only` option below.
+    void forward();
     // forward() with a HIP event between layers; ms[i] = time of layer i.
     void forward_timed(std::vector<float> &ms);
+    // Recurrent nets only, [net] key `last_step_only=1` (a key the reference ignores): the layers after
+    // the last LSTM see only the rows of the final time step (B rows instead of T*B), i.e. the output
+    // projection and softmax are computed for the last step alone.
+    bool last_step_only;
 
 protected:
     void init_network(const std::string m_network_config);
@@ -88,6 +94,8 @@ protected:
 
 private:
     void build(class config_t &config);
+    void run_layer(unsigned i);
+    int first_after_lstm;      // index of the first layer after the last LSTM, -1 if none
     unsigned batch_override;
     bool is_recurrent;
     std::vector<void*> events;

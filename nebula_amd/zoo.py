@@ -68,8 +68,12 @@ def resnet50_cfg(batch=64, activation="relu"):
     return s
 
 
-def lstm_cfg(batch=64, time_steps=64, input_size=1024, hidden=1024, layers=2, classes=10000):
+def lstm_cfg(batch=64, time_steps=64, input_size=1024, hidden=1024, layers=2, classes=10000, last_step_only=False):
+    """last_step_only: project and softmax the final time step only (a [net] key the reference ignores;
+    the reference itself projects all T*B rows)."""
     s = "[net]\nbatch=%d\ninput_size=%d\ntime_steps=%d\n" % (batch, input_size, time_steps)
+    if last_step_only:
+        s += "last_step_only=1\n"
     for _ in range(layers):
         s += "\n[lstm]\noutput=%d\nactivation=linear\n" % hidden
     s += _fc(classes, "linear") + _TAIL

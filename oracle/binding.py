@@ -306,6 +306,8 @@ def plan_network(cfg_text, batch=None):
             if "time_steps" in kv:
                 net["recurrent"] = True
                 net["time_steps"] = g("time_steps", 1)
+                # harness extension (a key the reference ignores): layers after the last LSTM see the final step only
+                net["last_step_only"] = bool(g("last_step_only", 0))
                 net["input_size"] = g("input_size", 0)
                 cur = (1, 1, 1, net["input_size"])
             else:
@@ -435,6 +437,11 @@ class OracleNet:
                           [wt[s + ".var"] for s in subs])
                 cur = lstm_forward(cur.reshape(T, -1, sp.I), [wt[s + ".weight"] for s in subs],
                                    [wt[s + ".bias"] for s in subs], bn, sp.act)
+                last_lstm = max(i for i, q in enumerate(self.specs) if q.kind == "lstm")
+                if self.net.get("last_step_only") and li == last_lstm:
+                    outs.append(cur)
+                    cur = cur[-1:]          # [1, B, H]: only the final step feeds the rest
+                    continue
             outs.append(cur)
         return outs
 

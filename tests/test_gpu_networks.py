@@ -178,3 +178,31 @@ def test_mini_resnet_against_oracle():
             assert rel(got, want[i].ravel()) <= TOL, (i, net.layer_info(i)["kind"], rel(got, want[i].ravel()))
         logits = net.output(net.num_layers - 2).reshape(4, -1)
         np.testing.assert_array_equal(logits.argmax(1), want[-2].reshape(4, -1).argmax(1))
+
+
+def test_lstm_last_step_only_against_oracle():
+    from nebula_amd import zoo
+    from nebula_amd.net import Network
+    print("CASE lstm last_step_only", flush=True)
+    T, B, I, H, Cn = 5, 6, 24, 64, 37
+    rng = np.random.default_rng(8)
+    for last in (False, True):
+        cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=I, hidden=H, layers=2, classes=Cn, last_step_only=last)
+        onet = ob.OracleNet(cfg)
+        blob = np.concatenate([rng.uniform(-1, 1, int(np.prod(sh))).astype(np.float32) / np.float32(np.sqrt(H))
+                               for _, _, sh in ob.weight_layout(onet.specs)])
+        onet.load_weights(blob)
+        x = rng.standard_normal((T, B, I)).astype(np.float32)
+        ob.use_custom_gemm()
+        want = onet.forward(x)
+        rows = B if last else T * B
+        assert want[3].shape == (rows, Cn)
+        with Network(cfg) as net:
+            net.load_weight_blob(blob)
+            net.set_input(x)
+            net.forward()
+            for i in (0, 1):
+                assert rel(net.output(i), want[i].ravel()) <= TOL
+            probs = net.output(3).reshape(T * B, Cn)[:rows]
+            assert rel(probs, want[3]) <= TOL
+            np.testing.assert_array_equal(probs.argmax(1), want[3].argmax(1))
