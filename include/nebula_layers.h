@@ -22,7 +22,9 @@ extern "C" {
 typedef struct nbl_net nbl_net;
 
 /* cfg: path of a network.cfg (is_text = 0) or its contents (is_text = 1).  batch_override > 0 replaces
- * the [net] section's batch=.  weight_path may be NULL or "" (load later with nbl_net_load_weights). */
+ * the [net] section's batch=.  weight_path may be NULL or "" (load later with nbl_net_load_weights).
+ * device < 0 builds a dry-run network: cfg parsing, shape inference, .wgh reading/writing and the
+ * queries below work without a GPU; anything that would compute fails with an error. */
 int nbl_net_create(const char *cfg, int is_text, unsigned batch_override, int device,
                    const char *weight_path, nbl_net **out);
 int nbl_net_destroy(nbl_net *net);

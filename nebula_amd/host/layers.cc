@@ -37,7 +37,7 @@ layer_t::layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_lay
 }
 
 layer_t::~layer_t() {
-    if(owns_output && output_data_dev) nbl_free(network->ctx, output_data_dev);
+    if(owns_output && output_data_dev && network->ctx) nbl_free(network->ctx, output_data_dev);
     delete [] output_data;
 }
 
@@ -62,6 +62,7 @@ const float *layer_t::input_dev() const {
 }
 
 void layer_t::alloc_output() {
+    if(!network->ctx) return;          // dry-run network: shapes only
     const size_t bytes = sizeof(float) * (size_t)output_size * network->batch_size;
     nbl_check(network->ctx, nbl_malloc(network->ctx, (void**)&output_data_dev, bytes), "nbl_malloc(output)");
     nbl_check(network->ctx, nbl_fill_zero(network->ctx, output_data_dev, bytes), "nbl_fill_zero(output)");
@@ -142,6 +143,7 @@ void convolutional_layer_t::store_weight(std::fstream &m_weight_file) {
 }
 
 void convolutional_layer_t::pack() {
+    if(!network->ctx) return;          // dry-run network
     if(plan) { nbl_conv2d_plan_destroy(network->ctx, plan); plan = NULL; }
     nbl_check(network->ctx,
               nbl_conv2d_pack(network->ctx, weight.data(), bias.data(),
@@ -245,6 +247,7 @@ void connected_layer_t::weight_fields(std::vector<weight_field_t> &out) const {
 }
 
 void connected_layer_t::pack() {
+    if(!network->ctx) return;          // dry-run network
     if(plan) { nbl_fc_plan_destroy(network->ctx, plan); plan = NULL; }
     nbl_check(network->ctx,
               nbl_fc_pack(network->ctx, weight.data(), bias.data(),
@@ -289,7 +292,7 @@ void pooling_layer_t::init(section_config_t m_section_config) {
     output_channel = input_channel;
     output_size    = output_height * output_width * output_channel;
     alloc_output();
-    if(layer_type == MAXPOOL_LAYER) {
+    if(layer_type == MAXPOOL_LAYER && network->ctx) {
         const size_t bytes = sizeof(unsigned) * (size_t)output_size * network->batch_size;
         nbl_check(network->ctx, nbl_malloc(network->ctx, (void**)&index_dev, bytes), "nbl_malloc(index)");
         nbl_check(network->ctx, nbl_fill_zero(network->ctx, index_dev, bytes), "nbl_fill_zero(index)");
@@ -454,6 +457,7 @@ void lstm_layer_t::weight_fields(std::vector<weight_field_t> &out) const {
 }
 
 void lstm_layer_t::pack() {
+    if(!network->ctx) return;          // dry-run network
     if(plan) { nbl_lstm_plan_destroy(network->ctx, plan); plan = NULL; }
     connected_layer_t *order[8] = { input_gate_W, forget_gate_W, output_gate_W, cell_gate_W,
                                     input_gate_U, forget_gate_U, output_gate_U, cell_gate_U };

@@ -66,6 +66,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
     last_step_only(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false) {
     run_type = TEST_RUN;
+    if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
     if(rc != NBL_OK) {
         std::ostringstream msg;
@@ -77,7 +78,7 @@ inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
 inference_net_t::~inference_net_t() {
     for(size_t i = layers.size(); i > 0; i--) delete layers[i - 1];
     for(size_t i = 0; i < events.size(); i++) (void)hipEventDestroy((hipEvent_t)events[i]);
-    if(input_data_dev) nbl_free(ctx, input_data_dev);
+    if(input_data_dev && ctx) nbl_free(ctx, input_data_dev);
     delete [] input_data;
     if(ctx) nbl_ctx_destroy(ctx);
 }
@@ -150,15 +151,17 @@ void inference_net_t::build(config_t &config) {
 }
 
 void inference_net_t::init_data(const std::string) {
-    if(input_data_dev) return;
+    if(input_data_dev || input_data) return;
     const size_t count = (size_t)batch_size * input_size;
     input_data = new float[count]();
+    if(!ctx) return;
     nbl_check(ctx, nbl_malloc(ctx, (void**)&input_data_dev, count * sizeof(float)), "nbl_malloc(input)");
     nbl_check(ctx, nbl_fill_zero(ctx, input_data_dev, count * sizeof(float)), "nbl_fill_zero(input)");
     // the first layer captured the (then NULL) input pointer lazily through input_dev(), nothing to patch
 }
 
 void inference_net_t::set_input(const float *host, size_t count) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     if(count != (size_t)batch_size * input_size) throw std::runtime_error("Error: input tensor has the wrong size");
     nbl_check(ctx, nbl_h2d(ctx, input_data_dev, host, count * sizeof(float)), "nbl_h2d(input)");
 }
@@ -191,10 +194,12 @@ void inference_net_t::run_layer(unsigned i) {
 }
 
 void inference_net_t::forward() {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     for(unsigned i = 0; i < num_layers; i++) run_layer(i);
 }
 
 void inference_net_t::forward_timed(std::vector<float> &ms) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     hipStream_t stream = (hipStream_t)nbl_ctx_stream(ctx);
     while(events.size() < (size_t)num_layers + 1) {
         hipEvent_t e;
