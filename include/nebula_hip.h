@@ -84,6 +84,15 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
                     unsigned C, unsigned H, unsigned W, unsigned F,
                     unsigned ksize, unsigned stride, unsigned pad, int act, nbl_conv_plan **out);
 int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B);
+/* Convolution with the following [shortcut] layer in its epilogue: y = post_act(act(conv(x)) + conn'),
+ * conn' = conn cropped to the common channel/height/width box and sampled with stride
+ * max(1, conn_w / OW), exactly what convolutional_layer_t::_forward_() followed by
+ * shortcut_layer_t::_forward_() compute (models/layers/shortcut_layer.cu:27-52, common/utils.cc:28-60)
+ * in the same float operations and order, without writing and re-reading the convolution's output.
+ * conn_dev is [B][conn_c][conn_h][conn_w]; y_dev is [B][F][OH][OW] and must not alias conn_dev.
+ * An up-sampling shortcut (OW / conn_w > 1) is not fused: NBL_EUNSUPPORTED. */
+int nbl_conv2d_shortcut_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, const float *conn_dev,
+                            unsigned conn_c, unsigned conn_h, unsigned conn_w, float *y_dev, unsigned B, int post_act);
 int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *plan);
 /* Algorithmic FLOP of one forward at batch B (2*B*F*OH*OW*C*k*k) and the output dims. */
 int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, double *flop_per_image);

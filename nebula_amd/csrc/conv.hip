@@ -19,6 +19,7 @@
 #include "nbl_internal.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -37,6 +38,8 @@ struct ConvArgs {
     unsigned x_bytes;
     int act, has_scale;
     int tiles_m, tiles_n;
+    // optional fused shortcut: y = post_act(act(conv) + res'), res' = res cropped/strided as common/utils.cc:28-60
+    const float *res; int res_c, res_hw, res_w, res_stride, res_box_h, res_box_w, post_act;
 };
 
 struct PixelCoord { int xbase; int ih0; int iw0; };
@@ -89,8 +92,9 @@ enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
        GATHER_1X1_VEC4 = 2  // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
 };
 
-template<int MT, int NT, int WAVES_M, int WAVES_N, int GATHER, bool FAST_ACT>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N)
+// OCC = blocks the register budget must leave room for on a CU (the persistent grid is sized with it)
+template<int MT, int NT, int WAVES_M, int WAVES_N, int OCC, int GATHER, bool FAST_ACT>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC)
 void conv_igemm_kernel(const ConvArgs a) {
     constexpr int BK = CONV_BK;
     constexpr int NTHREADS = 64 * WAVES_M * WAVES_N;
@@ -113,10 +117,11 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     const int half = lane >> 5, l32 = lane & 31;
 
-    // m-tile fastest: the blocks that share one pixel tile run next to each other.
-    const int tile = blockIdx.x;
-    const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
-    const int m0 = tm * BM, n0 = tn * BN;
+    // Persistent blocks: block b works through output tiles b, b + gridDim.x, ... (m-tile fastest, so
+    // the blocks that share one pixel tile run next to each other).  The load side runs two k-tiles
+    // ahead of the MFMAs and simply crosses into the next output tile, so a tile's first loads overlap
+    // the previous tile's last MFMAs, and its epilogue stores drain while the next tile is multiplied.
+    const int total_tiles = a.tiles_m * a.tiles_n;
 
     const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.x, a.x_bytes);
     const int ncol = tid % NCOLS;
@@ -125,16 +130,29 @@ void conv_igemm_kernel(const ConvArgs a) {
     // VEC4 mode: four pixel columns per thread, k rows strided by KGROUPS, no table (offset = k * H*W).
     const int kgroup = VEC4 ? tid / NCOLS : __builtin_amdgcn_readfirstlane(tid / NCOLS);
     const int krow0 = VEC4 ? kgroup : kgroup * RB;
-    // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past the
-    // last pixel re-reads the last group (its results are never stored), a row past the last patch row
-    // re-reads the last row and is zeroed when the tile is written to LDS.
-    const int ncol_first = VEC4 ? min(n0 + ncol * 4, a.N - 4) : n0 + ncol;
-    const PixelCoord px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
-    // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
-    const unsigned xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
-    const float *__restrict__ xpix = a.x + (VEC4 ? px.xbase : 0);
 
-    // Two register stages: the loads of tile t+2 are issued while tile t is multiplied and tile t+1 is
+    // ---- load side state: which output tile and k-tile the next global loads belong to ----
+    int ld_tile = blockIdx.x, ld_kt = 0, ld_m0 = 0;
+    PixelCoord px;
+    unsigned xoff = 0;
+    const float *__restrict__ xpix = a.x;
+    auto ld_set_tile = [&](int tile) {
+        // past the block's last tile (pipeline tail) the loads repeat the last real tile; they are never used
+        const int t = tile < total_tiles ? tile : total_tiles - 1;
+        const int tm = t % a.tiles_m, tn = t / a.tiles_m;
+        ld_m0 = tm * BM;
+        const int n0 = tn * BN;
+        // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past
+        // the last pixel re-reads the last group (its results are never stored), a row past the last patch
+        // row re-reads the last row and is zeroed when the tile is written to LDS.
+        const int ncol_first = VEC4 ? min(n0 + ncol * 4, a.N - 4) : n0 + ncol;
+        px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
+        // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
+        xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
+        xpix = a.x + (VEC4 ? px.xbase : 0);
+    };
+
+    // Two register stages: the loads of k-tile t+2 are issued while k-tile t is multiplied and t+1 is
     // still in flight, so every global load has two k-tiles of MFMA time to arrive.
     struct Stage {
         float b[VEC4 ? 1 : RB];
@@ -143,7 +161,7 @@ void conv_igemm_kernel(const ConvArgs a) {
         unsigned kvalid;
     };
     Stage st0, st1;
-    int2 ke[VEC4 ? 1 : RB];  // table entries of the next tile to gather
+    int2 ke[VEC4 ? 1 : RB];  // table entries of the next k-tile to gather
 
     auto load_ktab = [&](int kt) {
         if(!VEC4) {
@@ -152,9 +170,7 @@ void conv_igemm_kernel(const ConvArgs a) {
             for(int r = 0; r < RB; r++) ke[r] = tp[r];
         }
     };
-    // kt may run past the last tile (the pipeline tail): the weight tile index is clamped, the table has
-    // all-padding tiles behind the last one, and the VEC4 path clamps its row; such a tile is never used.
-    auto load_tile = [&](Stage &st, int kt, int nkt) {
+    auto load_tile = [&](Stage &st, int kt) {
         if(VEC4) {
             st.kvalid = 0;
             #pragma unroll
@@ -173,7 +189,7 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.b[r] = buf_load(xres, off);
             }
         }
-        const float *__restrict__ wtile = a.wp + (size_t)min(kt, nkt - 1) * BK * a.Mp + m0;
+        const float *__restrict__ wtile = a.wp + (size_t)kt * BK * a.Mp + ld_m0;
         {
             const int row = tid / (BM / 4), col4 = tid % (BM / 4);
             if(A_VEC >= NTHREADS || tid < A_VEC)
@@ -185,6 +201,18 @@ void conv_igemm_kernel(const ConvArgs a) {
             if(A_VEC >= 2 * NTHREADS || v < A_VEC)
                 st.a1 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
         }
+    };
+    const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
+    // issue the loads of the next k-tile in sequence and move the cursor (into the next output tile
+    // after the last k-tile of this one); the table entries of the k-tile after it follow
+    auto ld_next = [&](Stage &st) {
+        load_tile(st, ld_kt);
+        if(++ld_kt == nkt) {
+            ld_kt = 0;
+            ld_tile += gridDim.x;
+            ld_set_tile(ld_tile);
+        }
+        load_ktab(ld_kt);
     };
     auto store_tile = [&](const Stage &st, int buf) {
         if(VEC4) {
@@ -208,12 +236,6 @@ void conv_igemm_kernel(const ConvArgs a) {
     };
 
     floatx16 acc[MT][NT];
-    #pragma unroll
-    for(int i = 0; i < MT; i++)
-        #pragma unroll
-        for(int j = 0; j < NT; j++)
-            #pragma unroll
-            for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     // Rows and columns are dealt to the MFMA tiles of a wave interleaved: tile i of the wave holds rows
     // l*MT + i (l = 0..31) and tile j holds columns l*NT + j.  A lane therefore finds the MT (NT)
@@ -221,6 +243,8 @@ void conv_igemm_kernel(const ConvArgs a) {
     // compile-time offset, and in the epilogue it owns NT adjacent pixels of each of its rows.
     const float *a_lane = &As[0][half][wm * MT * 32 + l32 * MT];
     const float *b_lane = &Bs[0][half][wn * NT * 32 + l32 * NT];
+    // all MFMAs of one resident k-tile; the operands of k-step ks+1 are fetched from LDS before the
+    // MFMAs of k-step ks are issued
     auto compute_tile = [&](int buf) {
         const float *ap = a_lane + buf * (BK * LDA), *bp = b_lane + buf * (BK * LDB);
         float av[2][MT], bv[2][NT];
@@ -247,106 +271,167 @@ void conv_igemm_kernel(const ConvArgs a) {
         }
     };
 
-    const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
-    st0.a0 = st0.a1 = st1.a0 = st1.a1 = make_float4(0.f, 0.f, 0.f, 0.f);
-    load_ktab(0);
-    load_tile(st0, 0, nkt);
-    load_ktab(1);
-    load_tile(st1, 1, nkt);
-    load_ktab(2);
-    store_tile(st0, 0);
-    __syncthreads();
-
-    for(int kt = 0; kt < nkt; kt += 2) {
-        // tile kt is in LDS buffer 0, tile kt+1 is in flight in stage 1
-#ifndef NBL_EXP_NO_GLOBAL
-        load_tile(st0, kt + 2, nkt);
-        load_ktab(kt + 3);
-#endif
-        compute_tile(0);
-#ifndef NBL_EXP_NO_LDSWRITE
-        store_tile(st1, 1);
-#endif
-#ifndef NBL_EXP_NO_BARRIER
-        __syncthreads();
-#endif
-        // tile kt+1 is in LDS buffer 1, tile kt+2 is in flight in stage 0
-#ifndef NBL_EXP_NO_GLOBAL
-        load_tile(st1, kt + 3, nkt);
-        load_ktab(kt + 4);
-#endif
-        compute_tile(1);
-#ifndef NBL_EXP_NO_LDSWRITE
-        store_tile(st0, 0);
-#endif
-#ifndef NBL_EXP_NO_BARRIER
-        __syncthreads();
-#endif
-    }
-
-    // Epilogue: y = act(acc * g[f] + b[f]).  Accumulator register r of a 32x32 MFMA tile holds tile row
-    // 8*(r/4) + 4*(lane/32) + r%4 and tile column lane%32; with the interleaving above that is
-    // filter row*MT + i and pixel (lane%32)*NT + j of the wave's sub-tile.
-    const int nbase = n0 + wn * NT * 32 + l32 * NT;
-    if(nbase >= a.N) return;
-    const int b0 = nbase / a.OHW, pix0 = nbase - b0 * a.OHW;
-    // the NT pixels of this lane are contiguous in memory when they sit in one image; then (and when the
-    // address is 8-byte aligned) a pair is written as one 64-bit store
-    const bool pair_ok = NT == 2 && pix0 + 1 < a.OHW && ((pix0 | a.OHW) & 1) == 0;
-    // Per-filter constants first, all loads in flight together: for each group q of four accumulator
-    // registers the lane's filters f = fq + rr*MT + i (rr = r%4) are 4*MT consecutive entries of the
-    // (zero padded) g and b vectors.
-    float gq[4][4 * MT], bq[4][4 * MT];
-    #pragma unroll
-    for(int q = 0; q < 4; q++) {
-        const int fq = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT;
+    // Epilogue of one finished output tile: y = act(acc * g[f] + b[f]) (+ fused shortcut).
+    // Accumulator register r of a 32x32 MFMA tile holds tile row 8*(r/4) + 4*(lane/32) + r%4 and tile
+    // column lane%32; with the interleaving above that is filter row*MT + i and pixel (lane%32)*NT + j
+    // of the wave's sub-tile.
+    auto epilogue = [&](int tile) {
+        const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
+        const int m0 = tm * BM, n0 = tn * BN;
+        const int nbase = n0 + wn * NT * 32 + l32 * NT;
+        if(nbase >= a.N) return;
+        const int b0 = nbase / a.OHW, pix0 = nbase - b0 * a.OHW;
+        // the NT pixels of this lane are contiguous in memory when they sit in one image; then (and when
+        // the address is 8-byte aligned) a pair is written as one 64-bit store
+        const bool pair_ok = NT == 2 && pix0 + 1 < a.OHW && ((pix0 | a.OHW) & 1) == 0;
+        float *__restrict__ ybase = a.y + (size_t)b0 * a.F * a.OHW + pix0;
+        // fused shortcut: per pixel of this lane, where its residual sits and whether it has one
+        int roff[NT]; bool rok[NT];
         #pragma unroll
-        for(int v = 0; v < MT; v++) {
-            const float4 bb = *reinterpret_cast<const float4*>(a.b + fq + 4 * v);
-            bq[q][4 * v] = bb.x; bq[q][4 * v + 1] = bb.y; bq[q][4 * v + 2] = bb.z; bq[q][4 * v + 3] = bb.w;
-            if(a.has_scale) {
-                const float4 gg = *reinterpret_cast<const float4*>(a.g + fq + 4 * v);
-                gq[q][4 * v] = gg.x; gq[q][4 * v + 1] = gg.y; gq[q][4 * v + 2] = gg.z; gq[q][4 * v + 3] = gg.w;
-            }
-        }
-    }
-    float *__restrict__ ybase = a.y + (size_t)b0 * a.F * a.OHW + pix0;
-    #pragma unroll
-    for(int i = 0; i < MT; i++) {
-        #pragma unroll
-        for(int r = 0; r < 16; r++) {
-            const int q = r >> 2, e = (r & 3) * MT + i;
-            const int f = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT + e;
-            if(f >= a.F) continue;
-            const float bf = bq[q][e], gf = a.has_scale ? gq[q][e] : 1.0f;
-            float v[NT];
+        for(int j = 0; j < NT; j++) { roff[j] = 0; rok[j] = false; }
+        if(a.res) {
             #pragma unroll
             for(int j = 0; j < NT; j++) {
-                float t = acc[i][j][r];
-                t = a.has_scale ? t * gf + bf : t + bf;
-                if(FAST_ACT) {
-                    // relu / linear / leaky / relie: no transcendental, same predicates as nbl_act_apply
-                    if(a.act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
-                    else if(a.act == NBL_ACT_LEAKY) t = t > 0.0f ? t : (float)(0.1 * (double)t);
-                    else if(a.act == NBL_ACT_RELIE) t = t > 0.0f ? t : (float)(0.01 * (double)t);
-                } else {
-                    t = nbl_act_apply(a.act, t);
+                const int n = nbase + j;
+                if(n < a.N) {
+                    const int b = n / a.OHW, pix = n - b * a.OHW;
+                    const int h = pix / a.OW, w = pix - h * a.OW;
+                    rok[j] = h < a.res_box_h && w < a.res_box_w;
+                    roff[j] = b * a.res_c * a.res_hw + h * a.res_stride * a.res_w + w * a.res_stride;
                 }
-                v[j] = t;
             }
-            if(pair_ok) {
-                *reinterpret_cast<float2*>(ybase + (size_t)f * a.OHW) = make_float2(v[0], v[NT - 1]);
-            } else {
+        }
+        const float *__restrict__ res = a.res;
+        // residuals of a lane's NT pixels are adjacent when the shortcut keeps the spatial size: one 64-bit load
+        const bool res_pair = res && pair_ok && rok[0] && rok[NT - 1] && roff[NT - 1] == roff[0] + 1 &&
+                              ((roff[0] | a.res_hw) & 1) == 0;
+        // One group of four accumulator registers (4*MT consecutive filters of this lane) at a time, so the
+        // epilogue's temporaries stay few next to the load stages that are live across it: the group's
+        // per-filter constants (4*MT consecutive entries of the zero-padded g and b vectors) and residuals
+        // are fetched together, then combined and stored.
+        #pragma unroll
+        for(int q = 0; q < 4; q++) {
+            const int fq = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT;
+            if(fq >= a.F) continue;
+            float gq[4 * MT], bq[4 * MT];
+            #pragma unroll
+            for(int v = 0; v < MT; v++) {
+                const float4 bb = *reinterpret_cast<const float4*>(a.b + fq + 4 * v);
+                bq[4 * v] = bb.x; bq[4 * v + 1] = bb.y; bq[4 * v + 2] = bb.z; bq[4 * v + 3] = bb.w;
+                if(a.has_scale) {
+                    const float4 gg = *reinterpret_cast<const float4*>(a.g + fq + 4 * v);
+                    gq[4 * v] = gg.x; gq[4 * v + 1] = gg.y; gq[4 * v + 2] = gg.z; gq[4 * v + 3] = gg.w;
+                }
+            }
+            float rv[4 * MT][NT];
+            if(res) {
                 #pragma unroll
-                for(int j = 0; j < NT; j++) {
-                    const int n = nbase + j;
-                    if(n < a.N) {
-                        const int b = n / a.OHW, pix = n - b * a.OHW;
-                        a.y[((size_t)b * a.F + f) * a.OHW + pix] = v[j];
+                for(int e = 0; e < 4 * MT; e++) {
+                    const int f = fq + e;
+                    #pragma unroll
+                    for(int j = 0; j < NT; j++) rv[e][j] = 0.0f;
+                    if(f < a.F && f < a.res_c) {
+                        if(res_pair) {
+                            const float2 t = *reinterpret_cast<const float2*>(res + roff[0] + f * a.res_hw);
+                            rv[e][0] = t.x; rv[e][NT - 1] = t.y;
+                        } else {
+                            #pragma unroll
+                            for(int j = 0; j < NT; j++) if(rok[j]) rv[e][j] = res[roff[j] + f * a.res_hw];
+                        }
+                    }
+                }
+            }
+            #pragma unroll
+            for(int rr = 0; rr < 4; rr++) {
+                #pragma unroll
+                for(int i = 0; i < MT; i++) {
+                    const int e = rr * MT + i, r = q * 4 + rr;
+                    const int f = fq + e;
+                    if(f >= a.F) continue;
+                    const float bf = bq[e], gf = a.has_scale ? gq[e] : 1.0f;
+                    float v[NT];
+                    #pragma unroll
+                    for(int j = 0; j < NT; j++) {
+                        float t = acc[i][j][r];
+                        t = a.has_scale ? t * gf + bf : t + bf;
+                        if(FAST_ACT) {
+                            // relu / linear / leaky / relie: no transcendental, same predicates as nbl_act_apply
+                            if(a.act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
+                            else if(a.act == NBL_ACT_LEAKY) t = t > 0.0f ? t : (float)(0.1 * (double)t);
+                            else if(a.act == NBL_ACT_RELIE) t = t > 0.0f ? t : (float)(0.01 * (double)t);
+                        } else {
+                            t = nbl_act_apply(a.act, t);
+                        }
+                        v[j] = t;
+                    }
+                    if(res) {
+                        #pragma unroll
+                        for(int j = 0; j < NT; j++) {
+                            // an element without a residual keeps its value: adding a 0.0f placeholder would turn -0 into +0
+                            float t = (f < a.res_c && rok[j]) ? __fadd_rn(v[j], rv[e][j]) : v[j];
+                            if(FAST_ACT) {
+                                if(a.post_act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
+                                else if(a.post_act == NBL_ACT_LEAKY) t = t > 0.0f ? t : (float)(0.1 * (double)t);
+                                else if(a.post_act == NBL_ACT_RELIE) t = t > 0.0f ? t : (float)(0.01 * (double)t);
+                            } else {
+                                t = nbl_act_apply(a.post_act, t);
+                            }
+                            v[j] = t;
+                        }
+                    }
+                    if(pair_ok) {
+                        *reinterpret_cast<float2*>(ybase + (size_t)f * a.OHW) = make_float2(v[0], v[NT - 1]);
+                    } else {
+                        #pragma unroll
+                        for(int j = 0; j < NT; j++) {
+                            const int n = nbase + j;
+                            if(n < a.N) {
+                                const int b = n / a.OHW, pix = n - b * a.OHW;
+                                a.y[((size_t)b * a.F + f) * a.OHW + pix] = v[j];
+                            }
+                        }
                     }
                 }
             }
         }
+    };
+
+    // ---- pipeline start: k-tiles 0 and 1 of the block's first output tile ----
+    st0.a0 = st0.a1 = st1.a0 = st1.a1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    ld_set_tile(ld_tile);
+    load_ktab(0);
+    ld_next(st0);
+    ld_next(st1);
+    store_tile(st0, 0);
+    __syncthreads();
+
+    for(int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+        #pragma unroll
+        for(int i = 0; i < MT; i++)
+            #pragma unroll
+            for(int j = 0; j < NT; j++)
+                #pragma unroll
+                for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+        for(int kt = 0; kt < nkt; kt += 2) {
+            // k-tile kt is in LDS buffer 0, kt+1 is in flight in stage 1
+#ifndef NBL_EXP_NO_GLOBAL
+            ld_next(st0);
+#endif
+            compute_tile(0);
+            store_tile(st1, 1);
+            __syncthreads();
+            // k-tile kt+1 is in LDS buffer 1, kt+2 (possibly the next output tile's first) is in flight in stage 0
+#ifndef NBL_EXP_NO_GLOBAL
+            ld_next(st1);
+#endif
+            compute_tile(1);
+            store_tile(st0, 0);
+            __syncthreads();
+        }
+#ifdef NBL_EXP_NO_EPILOGUE
+        if(acc[0][0][0] != 12345.678f) continue;
+#endif
+        epilogue(tile);
     }
 }
 
@@ -378,22 +463,23 @@ std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, uns
 
 typedef void (*ConvKernel)(const ConvArgs);
 // kernel[gather mode][any activation ? 1 : 0]
-struct Variant { int bm, bn, threads; ConvKernel kernel[3][2]; const char *name; };
+struct Variant { int bm, bn, threads, blocks_per_cu; ConvKernel kernel[3][2]; const char *name; };
 
-#define NBL_CONV_VARIANT(MT, NT, WM, WN, NAME) \
-    { MT * 32 * WM, NT * 32 * WN, 64 * WM * WN, \
-      { { conv_igemm_kernel<MT, NT, WM, WN, GATHER_PADDED, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_PADDED, false> }, \
-        { conv_igemm_kernel<MT, NT, WM, WN, GATHER_NOPAD, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_NOPAD, false> }, \
-        { conv_igemm_kernel<MT, NT, WM, WN, GATHER_1X1_VEC4, true>, conv_igemm_kernel<MT, NT, WM, WN, GATHER_1X1_VEC4, false> } }, \
+// blocks_per_cu: resident blocks per CU (register- and LDS-limited), the size of the persistent grid
+#define NBL_CONV_VARIANT(MT, NT, WM, WN, OCC, NAME) \
+    { MT * 32 * WM, NT * 32 * WN, 64 * WM * WN, OCC, \
+      { { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_PADDED, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_PADDED, false> }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_NOPAD, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_NOPAD, false> }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, false> } }, \
       NAME }
 
 const Variant VARIANTS[] = {
-    NBL_CONV_VARIANT(2, 2, 2, 2, "128x128"),
-    NBL_CONV_VARIANT(2, 2, 1, 4, "64x256"),
-    NBL_CONV_VARIANT(3, 2, 1, 4, "96x256"),
-    NBL_CONV_VARIANT(1, 2, 2, 2, "64x128"),
-    NBL_CONV_VARIANT(1, 1, 2, 2, "64x64"),
-    NBL_CONV_VARIANT(2, 1, 2, 2, "128x64"),
+    NBL_CONV_VARIANT(2, 2, 2, 2, 3, "128x128"),
+    NBL_CONV_VARIANT(2, 2, 1, 4, 2, "64x256"),
+    NBL_CONV_VARIANT(3, 2, 1, 4, 2, "96x256"),
+    NBL_CONV_VARIANT(1, 2, 2, 2, 4, "64x128"),
+    NBL_CONV_VARIANT(1, 1, 2, 2, 6, "64x64"),
+    NBL_CONV_VARIANT(2, 1, 2, 2, 4, "128x64"),
 };
 constexpr int NUM_VARIANTS = sizeof(VARIANTS) / sizeof(VARIANTS[0]);
 
@@ -406,6 +492,7 @@ struct nbl_conv_plan {
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
     bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
+    bool persistent;            // blocks loop over several output tiles instead of taking exactly one (off: measured slower)
 };
 
 namespace {
@@ -457,7 +544,8 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->K = C * ksize * ksize;
     p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
-    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false; p->tuned_batch = 0; p->tuned_variant = -1;
+    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false; p->persistent = false;
+    if(const char *e = getenv("NBL_CONV_PERSISTENT")) p->persistent = atoi(e) != 0; p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL;
 
     // [F][K] -> [Kp][Mp], zero padded
@@ -505,7 +593,10 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
     return NBL_OK;
 }
 
-static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v) {
+struct ConvResidual { const float *res; unsigned c, h, w; int post_act; };
+
+static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v,
+                       const ConvResidual *rs) {
     const size_t in_elems = (size_t)B * p->C * p->H * p->W;
     const size_t npix = (size_t)B * p->OH * p->OW;
     const Variant &var = VARIANTS[v];
@@ -522,13 +613,32 @@ static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev,
         return nbl_fail(ctx, NBL_EINVAL, "nbl_conv2d_fwd: internal: tile %s overruns the packed weights", var.name);
     const size_t blocks = (size_t)a.tiles_m * a.tiles_n;
     if(blocks >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
-    const bool fast_act = p->act == NBL_ACT_RELU || p->act == NBL_ACT_LINEAR || p->act == NBL_ACT_LEAKY ||
-                          p->act == NBL_ACT_RELIE;
+    bool fast_act = p->act == NBL_ACT_RELU || p->act == NBL_ACT_LINEAR || p->act == NBL_ACT_LEAKY ||
+                    p->act == NBL_ACT_RELIE;
+    a.res = NULL; a.res_c = a.res_hw = a.res_w = a.res_stride = a.res_box_h = a.res_box_w = 0; a.post_act = NBL_ACT_LINEAR;
+    if(rs) {
+        // stride / crop rule of the shortcut layer (common/utils.cc:32-40); up-sampling is not fused
+        a.res = rs->res; a.res_c = (int)rs->c; a.res_hw = (int)(rs->h * rs->w); a.res_w = (int)rs->w;
+        a.res_stride = rs->w / p->OW > 1 ? (int)(rs->w / p->OW) : 1;
+        a.res_box_h = (int)(rs->h < p->OH ? rs->h : p->OH);
+        a.res_box_w = (int)(rs->w < p->OW ? rs->w : p->OW);
+        a.post_act = rs->post_act;
+        fast_act = fast_act && (rs->post_act == NBL_ACT_RELU || rs->post_act == NBL_ACT_LINEAR ||
+                                rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE);
+    }
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
     if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
        !p->force_scalar_gather)
         gather = GATHER_1X1_VEC4;
-    hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)blocks), dim3(var.threads), 0,
+    // persistent grid: as many blocks as stay resident (by registers and LDS), each looping over its tiles;
+    // the count is rounded so that every block gets the same number of tiles where possible
+    size_t grid = blocks;
+    const size_t resident = (size_t)ctx->num_cu * var.blocks_per_cu;
+    if(p->persistent && grid > resident) {
+        const size_t per_block = nbl_div_up_sz(blocks, resident);
+        grid = nbl_div_up_sz(blocks, per_block);
+    }
+    hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)grid), dim3(var.threads), 0,
                        ctx->stream, a);
     NBL_LAUNCH_CHECK(ctx, "conv_igemm_kernel");
     return NBL_OK;
@@ -537,7 +647,8 @@ static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev,
 // Tile search on the device: every tile shape runs the real problem twice and the faster second run
 // wins.  Block-count quantisation against the number of resident blocks decides more than any static
 // rule predicts, so the shapes are measured once per (layer, batch) and the result is kept in the plan.
-static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B) {
+static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
+                     const ConvResidual *rs) {
     hipEvent_t e0, e1;
     NBL_HIP(ctx, hipEventCreate(&e0));
     hipError_t err = hipEventCreate(&e1);
@@ -547,9 +658,9 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
     for(int v = 0; v < NUM_VARIANTS && rc == NBL_OK; v++) {
         if(nbl_div_up(p->F, VARIANTS[v].bm) * VARIANTS[v].bm > p->Mp) continue;
         float ms = 0.0f;
-        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v)) != NBL_OK) break;
+        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, rs)) != NBL_OK) break;
         if(hipEventRecord(e0, ctx->stream) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed"); break; }
-        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v)) != NBL_OK) break;
+        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, rs)) != NBL_OK) break;
         if(hipEventRecord(e1, ctx->stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
            hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "event timing failed"); break; }
         if(ms < best_ms) { best_ms = ms; best = v; }
@@ -560,10 +671,8 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
     return NBL_OK;
 }
 
-int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
-    if(!ctx) return NBL_EINVAL;
-    NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_conv2d_fwd: NULL argument");
-    if(B == 0) return NBL_OK;
+static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B,
+                        const ConvResidual *rs) {
     nbl_conv_plan *p = const_cast<nbl_conv_plan*>(plan);      // the tile-search result is a cache
     const size_t in_elems = (size_t)B * p->C * p->H * p->W, out_elems = (size_t)B * p->F * p->OH * p->OW;
     const size_t npix = (size_t)B * p->OH * p->OW;
@@ -574,11 +683,34 @@ int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, 
         if(p->tuned_batch != B) {
             // the search overwrites y with correct results several times; tiny problems are not worth it
             if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); }
-            else { int rc = conv_tune(ctx, p, x_dev, y_dev, B); if(rc != NBL_OK) return rc; }
+            else { int rc = conv_tune(ctx, p, x_dev, y_dev, B, rs); if(rc != NBL_OK) return rc; }
         }
         v = p->tuned_variant;
     }
-    return conv_launch(ctx, p, x_dev, y_dev, B, v);
+    return conv_launch(ctx, p, x_dev, y_dev, B, v, rs);
+}
+
+int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_conv2d_fwd: NULL argument");
+    if(B == 0) return NBL_OK;
+    return conv_forward(ctx, plan, x_dev, y_dev, B, NULL);
+}
+
+int nbl_conv2d_shortcut_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, const float *conn_dev,
+                            unsigned conn_c, unsigned conn_h, unsigned conn_w, float *y_dev, unsigned B, int post_act) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, plan && x_dev && y_dev && conn_dev, "nbl_conv2d_shortcut_fwd: NULL argument");
+    NBL_REQUIRE(ctx, conn_c && conn_h && conn_w, "nbl_conv2d_shortcut_fwd: zero dimension");
+    NBL_REQUIRE(ctx, nbl_act_valid(post_act), "nbl_conv2d_shortcut_fwd: undefined activation type %d", post_act);
+    NBL_REQUIRE(ctx, y_dev != conn_dev, "nbl_conv2d_shortcut_fwd: y must not alias conn");
+    if(plan->OW / conn_w > 1)
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: an up-sampling shortcut cannot be fused");
+    if((size_t)B * conn_c * conn_h * conn_w >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: residual tensor too large");
+    if(B == 0) return NBL_OK;
+    ConvResidual rs = { conn_dev, conn_c, conn_h, conn_w, post_act };
+    return conv_forward(ctx, plan, x_dev, y_dev, B, &rs);
 }
 
 int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigned W,

@@ -37,6 +37,7 @@ SIGNATURES = {
     "nbl_conv2d_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, _u, _u, _u, _u, _u, C.c_int,
                                   C.POINTER(_vp)]),
     "nbl_conv2d_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
+    "nbl_conv2d_shortcut_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u, _u, _vp, _u, C.c_int]),
     "nbl_conv2d_plan_destroy": (C.c_int, [_vp, _vp]),
     "nbl_conv2d_plan_info": (C.c_int, [_vp, C.POINTER(_u), C.POINTER(_u), C.POINTER(C.c_double)]),
     "nbl_conv2d_plan_set_variant": (C.c_int, [_vp, C.c_int]),
@@ -284,6 +285,14 @@ class ConvPlan:
         B = x.shape[0]
         y = out if out is not None else self.ctx.empty((B, self.F, self.OH, self.OW))
         self.ctx.check(lib().nbl_conv2d_fwd(self.ctx.h, self.p, x.ptr, y.ptr, B))
+        return y
+
+
+    def with_shortcut(self, x, conn, post_act="linear", out=None):
+        B = x.shape[0]
+        _, cc, ch, cw = conn.shape
+        y = out if out is not None else self.ctx.empty((B, self.F, self.OH, self.OW))
+        self.ctx.check(lib().nbl_conv2d_shortcut_fwd(self.ctx.h, self.p, x.ptr, conn.ptr, cc, ch, cw, y.ptr, B, ACT[post_act]))
         return y
 
 

@@ -71,7 +71,8 @@ void layer_t::alloc_output() {
 
 // ---- convolutional ---------------------------------------------------------------------------------
 convolutional_layer_t::convolutional_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type) :
-    layer_t(m_network, m_prev_layer, m_layer_type), batch_normalize(false), weight_size(0), plan(NULL) {}
+    layer_t(m_network, m_prev_layer, m_layer_type), batch_normalize(false), weight_size(0), plan(NULL),
+    fused_shortcut(NULL) {}
 
 convolutional_layer_t::~convolutional_layer_t() {
     if(plan) nbl_conv2d_plan_destroy(network->ctx, plan);
@@ -155,8 +156,29 @@ void convolutional_layer_t::pack() {
               "nbl_conv2d_pack");
 }
 
+bool convolutional_layer_t::fuse_with(shortcut_layer_t *m_shortcut) {
+    if(!m_shortcut || m_shortcut->prev_layer != this || fused_shortcut) return false;
+    layer_t *conn = m_shortcut->connection;
+    if(!conn || conn == this || output_width / conn->output_width > 1) return false;
+    if(owns_output && output_data_dev && network->ctx) nbl_free(network->ctx, output_data_dev);
+    owns_output = false;
+    output_data_dev = m_shortcut->output_data_dev;      // alias: nothing may read a stale buffer
+    fused_shortcut = m_shortcut;
+    m_shortcut->fused = true;
+    return true;
+}
+
 void convolutional_layer_t::_forward_() {
     if(!plan) throw std::runtime_error("Error: convolutional layer has no weights (init_weight not called)");
+    if(fused_shortcut) {
+        layer_t *conn = fused_shortcut->connection;
+        nbl_check(network->ctx,
+                  nbl_conv2d_shortcut_fwd(network->ctx, plan, input_dev(), conn->output_data_dev, conn->output_channel,
+                                          conn->output_height, conn->output_width, fused_shortcut->output_data_dev,
+                                          network->batch_size, (int)fused_shortcut->activation_type),
+                  "nbl_conv2d_shortcut_fwd");
+        return;
+    }
     nbl_check(network->ctx, nbl_conv2d_fwd(network->ctx, plan, input_dev(), output_data_dev, network->batch_size),
               "nbl_conv2d_fwd");
 }
@@ -309,7 +331,7 @@ void pooling_layer_t::_forward_() {
 
 // ---- shortcut --------------------------------------------------------------------------------------
 shortcut_layer_t::shortcut_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type) :
-    layer_t(m_network, m_prev_layer, m_layer_type), connection(NULL), hops(0) {}
+    layer_t(m_network, m_prev_layer, m_layer_type), connection(NULL), fused(false), hops(0) {}
 
 shortcut_layer_t::~shortcut_layer_t() {}
 
@@ -337,6 +359,7 @@ void shortcut_layer_t::init(section_config_t m_section_config) {
 }
 
 void shortcut_layer_t::_forward_() {
+    if(fused) return;          // already written by the preceding convolution
     nbl_check(network->ctx,
               nbl_shortcut_fwd(network->ctx, prev_layer->output_data_dev, connection->output_data_dev, output_data_dev,
                                network->batch_size, input_channel, input_height, input_width,

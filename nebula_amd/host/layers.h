@@ -77,12 +77,18 @@ public:
     void _forward_();
     void weight_fields(std::vector<weight_field_t> &out) const;
     double flop_per_image() const;
+    // Take over the [shortcut] layer that follows: this layer's kernel then adds the residual and applies
+    // the shortcut's activation in its epilogue and writes the shortcut's buffer; this layer's own output
+    // pointer becomes an alias of that buffer.  Returns false (and changes nothing) when the pair cannot
+    // be fused (up-sampling shortcut, or a shortcut whose source is this very layer).
+    bool fuse_with(class shortcut_layer_t *m_shortcut);
 private:
     void pack();
     bool batch_normalize;
     unsigned weight_size;
     std::vector<float> bias, weight, scale, rolling_mean, rolling_variance;
     nbl_conv_plan *plan;
+    class shortcut_layer_t *fused_shortcut;
 };
 
 // models/layers/connected_layer.h
@@ -129,8 +135,9 @@ public:
     void init_weight() {}
     void store_weight(std::fstream &) {}
     void _forward_();
+    layer_t *connection;       // the layer `hops` back whose output is added
+    bool fused;                // computed by the preceding convolution's epilogue; _forward_() does nothing
 private:
-    layer_t *connection;
     unsigned hops;
 };
 

@@ -64,7 +64,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    last_step_only(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false) {
+    last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
@@ -116,6 +116,7 @@ void inference_net_t::build(config_t &config) {
             sc.get_setting("width", &input_width);
             sc.get_setting("channels", &input_channel);
             sc.get_setting("batch", &batch_size);
+            sc.get_setting("fuse_shortcut", &fuse_shortcut);
             if(batch_override) batch_size = batch_override;
             input_size = input_height * input_width * input_channel;
             if(sc.exists("time_steps")) {
@@ -146,6 +147,10 @@ void inference_net_t::build(config_t &config) {
     }
     num_layers = (unsigned)layers.size();
     if(!output_layer && !layers.empty()) output_layer = layers.back();
+    if(fuse_shortcut)
+        for(unsigned i = 1; i < num_layers; i++)
+            if(layers[i]->layer_type == SHORTCUT_LAYER && layers[i - 1]->layer_type == CONVOLUTIONAL_LAYER)
+                static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
     for(unsigned i = 0; i < num_layers; i++)
         if(layers[i]->layer_type == LSTM_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
 }

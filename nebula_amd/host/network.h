@@ -85,6 +85,10 @@ public:
     // the last LSTM see only the rows of the final time step (B rows instead of T*B), i.e. the output
     // projection and softmax are computed for the last step alone.
     bool last_step_only;
+    // [net] key `fuse_shortcut=1` (a key the reference ignores): a convolution directly followed by a
+    // [shortcut] computes the residual add and the shortcut's activation in its own epilogue.  Same float
+    // operations in the same order; the convolution's pre-shortcut output is then never materialised.
+    bool fuse_shortcut;
 
 protected:
     void init_network(const std::string m_network_config);

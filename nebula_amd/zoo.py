@@ -7,8 +7,8 @@ convolutions, a 3x3/s2 maxpool with padding=0 and a 7x7/s7 average pool.
 """
 
 
-def _net(batch, h, w, c):
-    return "[net]\nbatch=%d\nheight=%d\nwidth=%d\nchannels=%d\n" % (batch, h, w, c)
+def _net(batch, h, w, c, extra=""):
+    return "[net]\nbatch=%d\nheight=%d\nwidth=%d\nchannels=%d\n%s" % (batch, h, w, c, extra)
 
 
 def _conv(filters, size, stride, padding, activation, bn=False):
@@ -54,8 +54,10 @@ def vgg16_cfg(batch=32):
     return s
 
 
-def resnet50_cfg(batch=64, activation="relu"):
-    s = _net(batch, 224, 224, 3)
+def resnet50_cfg(batch=64, activation="relu", fuse_shortcut=False):
+    """fuse_shortcut: let each block's last convolution add the residual in its epilogue (a [net] key the
+    reference ignores; results are bit-identical to the unfused network)."""
+    s = _net(batch, 224, 224, 3, "fuse_shortcut=1\n" if fuse_shortcut else "")
     s += _conv(64, 7, 2, 3, activation, bn=True) + _pool("maxpool", 3, 2, 0)
     for stage, (width, blocks) in enumerate(((64, 3), (128, 4), (256, 6), (512, 3))):
         for block in range(blocks):

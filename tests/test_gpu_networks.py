@@ -206,3 +206,44 @@ def test_lstm_last_step_only_against_oracle():
             probs = net.output(3).reshape(T * B, Cn)[:rows]
             assert rel(probs, want[3]) <= TOL
             np.testing.assert_array_equal(probs.argmax(1), want[3].argmax(1))
+
+
+def test_fused_shortcut_is_bit_identical():
+    """fuse_shortcut=1 moves the residual add into the convolution's epilogue: same operations, same order."""
+    from nebula_amd.net import Network
+    print("CASE fused shortcut", flush=True)
+    rng = np.random.default_rng(17)
+    fused_cfg = MINI_RESNET.replace("[net]\n", "[net]\nfuse_shortcut=1\n", 1)
+    onet = ob.OracleNet(MINI_RESNET)
+    blob = _random_weights(onet.specs, rng)
+    x = rng.standard_normal((4, 3, 32, 32)).astype(np.float32)
+    outs = []
+    for cfg in (MINI_RESNET, fused_cfg):
+        with Network(cfg) as net:
+            net.load_weight_blob(blob)
+            net.set_input(x)
+            net.forward()
+            kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
+            outs.append([net.output(i) for i in range(net.num_layers)])
+    for i, k in enumerate(kinds):
+        if k == "convolutional_layer" and i + 1 < len(kinds) and kinds[i + 1] == "shortcut_layer":
+            # the fused convolution's output pointer aliases the shortcut's buffer
+            np.testing.assert_array_equal(outs[1][i].view(np.uint32), outs[1][i + 1].view(np.uint32))
+            continue
+        np.testing.assert_array_equal(outs[0][i].view(np.uint32), outs[1][i].view(np.uint32), err_msg="layer %d %s" % (i, k))
+
+
+def test_fused_shortcut_on_golden_resnet(golden_dir):
+    from nebula_amd.net import Network
+    g = np.load(os.path.join(golden_dir, "resnet_shortcuts.npz"))
+    cfg = str(g["cfg"]).replace("[net]\n", "[net]\nfuse_shortcut=1\n", 1)
+    with Network(cfg) as net:
+        net.load_weight_blob(g["weights"])
+        net.set_input(g["input"])
+        net.forward()
+        for i in range(net.num_layers):
+            info = net.layer_info(i)
+            nxt = net.layer_info(i + 1)["kind"] if i + 1 < net.num_layers else ""
+            if info["kind"] == "convolutional_layer" and nxt == "shortcut_layer":
+                continue
+            assert rel(net.output(i), g["out_%02d" % i]) <= TOL, (i, info["kind"])
