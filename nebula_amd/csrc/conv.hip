@@ -20,6 +20,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <type_traits>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -40,7 +41,26 @@ struct ConvArgs {
     int tiles_m, tiles_n;
     // optional fused shortcut: y = post_act(act(conv) + res'), res' = res cropped/strided as common/utils.cc:28-60
     const float *res; int res_c, res_hw, res_w, res_stride, res_box_h, res_box_w, post_act;
+    // output (and residual, when there is one and it has the output's shape) addressable with 32-bit byte
+    // offsets and a cheap activation on both sides: full tiles may take the short epilogue
+    int short_epilogue;   // 0: no, 1: relu/linear only, 2: leaky or relie somewhere
 };
+
+// Activation of the short epilogue, written as selects on uniform flags so that the epilogue stays one
+// straight line of code the scheduler can interleave with its loads.  SLOPED = false knows relu and
+// linear; SLOPED = true adds leaky and relie with the predicate and double-precision product of
+// nbl_act_apply.
+template<bool SLOPED>
+__device__ __forceinline__ float conv_cheap_activation(float t, int act) {
+    const bool linear = act == NBL_ACT_LINEAR;
+    float neg = 0.0f;
+    if(SLOPED) {
+        const double slope = act == NBL_ACT_RELIE ? 0.01 : 0.1;
+        neg = act == NBL_ACT_RELU ? 0.0f : (float)(slope * (double)t);
+    }
+    const float r = t > 0.0f ? t : neg;
+    return linear ? t : r;
+}
 
 struct PixelCoord { int xbase; int ih0; int iw0; };
 
@@ -271,6 +291,52 @@ void conv_igemm_kernel(const ConvArgs a) {
         }
     };
 
+    // Short epilogue of a full tile whose rows are reached as base pointer + 32-bit byte offset: per row
+    // one integer add besides the arithmetic.  An instruction spent here is an instruction the matrix
+    // pipe waits for, which is most of what a layer with few patch rows does.  The per-filter scale is
+    // always applied (it is 1.0 where the layer has no batch normalisation, and acc * 1 + b rounds as
+    // acc + b does).
+    auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff) {
+        constexpr bool SLOPED = decltype(sloped)::value, RES = decltype(with_residual)::value;
+        typedef float __attribute__((ext_vector_type(NT))) pixvec;
+        const unsigned row_bytes = (unsigned)a.OHW * 4u;
+        char *__restrict__ yb = reinterpret_cast<char*>(a.y);
+        const char *__restrict__ rb = reinterpret_cast<const char*>(a.res);
+        const int act = a.act, post_act = a.post_act;
+        // per-filter constants one group of rows ahead of their use
+        float4 gv[2][MT], bv[2][MT];
+        auto load_constants = [&](int q) {
+            #pragma unroll
+            for(int u = 0; u < MT; u++) {
+                gv[q & 1][u] = *reinterpret_cast<const float4*>(a.g + f_lane + q * 8 * MT + 4 * u);
+                bv[q & 1][u] = *reinterpret_cast<const float4*>(a.b + f_lane + q * 8 * MT + 4 * u);
+            }
+        };
+        load_constants(0);
+        #pragma unroll
+        for(int q = 0; q < 4; q++) {
+            if(q + 1 < 4) load_constants(q + 1);
+            pixvec rv[4 * MT];
+            if(RES) {
+                #pragma unroll
+                for(int e = 0; e < 4 * MT; e++)
+                    rv[e] = *reinterpret_cast<const pixvec*>(rb + (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes));
+            }
+            #pragma unroll
+            for(int e = 0; e < 4 * MT; e++) {
+                const int rr = e / MT, i = e % MT;
+                const float ge = gv[q & 1][e / 4][e % 4], be = bv[q & 1][e / 4][e % 4];
+                pixvec o;
+                #pragma unroll
+                for(int j = 0; j < NT; j++) {
+                    o[j] = conv_cheap_activation<SLOPED>(__builtin_fmaf(acc[i][j][q * 4 + rr], ge, be), act);
+                    if(RES) o[j] = conv_cheap_activation<SLOPED>(__fadd_rn(o[j], rv[e][j]), post_act);
+                }
+                *reinterpret_cast<pixvec*>(yb + (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes)) = o;
+            }
+        }
+    };
+
     // Epilogue of one finished output tile: y = act(acc * g[f] + b[f]) (+ fused shortcut).
     // Accumulator register r of a 32x32 MFMA tile holds tile row 8*(r/4) + 4*(lane/32) + r%4 and tile
     // column lane%32; with the interleaving above that is filter row*MT + i and pixel (lane%32)*NT + j
@@ -281,6 +347,23 @@ void conv_igemm_kernel(const ConvArgs a) {
         const int nbase = n0 + wn * NT * 32 + l32 * NT;
         if(nbase >= a.N) return;
         const int b0 = nbase / a.OHW, pix0 = nbase - b0 * a.OHW;
+        // Short epilogue: every filter row of the tile exists, the lane's NT pixels are one aligned
+        // vector (OH*OW even keeps pairs inside one image), and rows are reached as base pointer +
+        // 32-bit offset, so a row costs one integer add besides its arithmetic.  An instruction spent
+        // here is an instruction the matrix pipe waits for, which is what layers with few patch rows
+        // are made of.
+        if(a.short_epilogue && m0 + BM <= a.F && (NT == 1 || (a.OHW & 1) == 0)) {
+            const int f_lane = m0 + wm * MT * 32 + half * 4 * MT;
+            const unsigned yoff = ((unsigned)(b0 * a.F + f_lane) * (unsigned)a.OHW + (unsigned)pix0) * 4u;
+            if(a.short_epilogue == 1) {
+                if(a.res) short_epilogue(std::false_type(), std::true_type(), f_lane, yoff);
+                else short_epilogue(std::false_type(), std::false_type(), f_lane, yoff);
+            } else {
+                if(a.res) short_epilogue(std::true_type(), std::true_type(), f_lane, yoff);
+                else short_epilogue(std::true_type(), std::false_type(), f_lane, yoff);
+            }
+            return;
+        }
         // the NT pixels of this lane are contiguous in memory when they sit in one image; then (and when
         // the address is 8-byte aligned) a pair is written as one 64-bit store
         const bool pair_ok = NT == 2 && pix0 + 1 < a.OHW && ((pix0 | a.OHW) & 1) == 0;
@@ -306,12 +389,35 @@ void conv_igemm_kernel(const ConvArgs a) {
         const bool res_pair = res && pair_ok && rok[0] && rok[NT - 1] && roff[NT - 1] == roff[0] + 1 &&
                               ((roff[0] | a.res_hw) & 1) == 0;
         // One group of four accumulator registers (4*MT consecutive filters of this lane) at a time, so the
-        // epilogue's temporaries stay few next to the load stages that are live across it: the group's
-        // per-filter constants (4*MT consecutive entries of the zero-padded g and b vectors) and residuals
-        // are fetched together, then combined and stored.
+        // epilogue's temporaries stay few next to the load stages that are live across it.  The group's
+        // per-filter constants are 4*MT consecutive entries of the zero-padded g and b vectors; the
+        // residuals of group q+1 are requested before group q is combined and stored, so residual reads
+        // and output writes overlap.
+        float rv[2][4 * MT][NT];
+        auto load_residuals = [&](int q, int slot) {
+            const int fq = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT;
+            #pragma unroll
+            for(int e = 0; e < 4 * MT; e++) {
+                const int f = fq + e;
+                #pragma unroll
+                for(int j = 0; j < NT; j++) rv[slot][e][j] = 0.0f;
+                if(f < a.F && f < a.res_c) {
+                    if(res_pair) {
+                        const float2 t = *reinterpret_cast<const float2*>(res + roff[0] + f * a.res_hw);
+                        rv[slot][e][0] = t.x; rv[slot][e][NT - 1] = t.y;
+                    } else {
+                        #pragma unroll
+                        for(int j = 0; j < NT; j++) if(rok[j]) rv[slot][e][j] = res[roff[j] + f * a.res_hw];
+                    }
+                }
+            }
+        };
+        if(res) load_residuals(0, 0);
         #pragma unroll
         for(int q = 0; q < 4; q++) {
             const int fq = m0 + wm * MT * 32 + (q * 8 + half * 4) * MT;
+            const int slot = q & 1;
+            if(res && q + 1 < 4) load_residuals(q + 1, slot ^ 1);
             if(fq >= a.F) continue;
             float gq[4 * MT], bq[4 * MT];
             #pragma unroll
@@ -321,24 +427,6 @@ void conv_igemm_kernel(const ConvArgs a) {
                 if(a.has_scale) {
                     const float4 gg = *reinterpret_cast<const float4*>(a.g + fq + 4 * v);
                     gq[4 * v] = gg.x; gq[4 * v + 1] = gg.y; gq[4 * v + 2] = gg.z; gq[4 * v + 3] = gg.w;
-                }
-            }
-            float rv[4 * MT][NT];
-            if(res) {
-                #pragma unroll
-                for(int e = 0; e < 4 * MT; e++) {
-                    const int f = fq + e;
-                    #pragma unroll
-                    for(int j = 0; j < NT; j++) rv[e][j] = 0.0f;
-                    if(f < a.F && f < a.res_c) {
-                        if(res_pair) {
-                            const float2 t = *reinterpret_cast<const float2*>(res + roff[0] + f * a.res_hw);
-                            rv[e][0] = t.x; rv[e][NT - 1] = t.y;
-                        } else {
-                            #pragma unroll
-                            for(int j = 0; j < NT; j++) if(rok[j]) rv[e][j] = res[roff[j] + f * a.res_hw];
-                        }
-                    }
                 }
             }
             #pragma unroll
@@ -353,7 +441,7 @@ void conv_igemm_kernel(const ConvArgs a) {
                     #pragma unroll
                     for(int j = 0; j < NT; j++) {
                         float t = acc[i][j][r];
-                        t = a.has_scale ? t * gf + bf : t + bf;
+                        t = __builtin_fmaf(t, gf, bf);   // gf = 1: rounds as t + bf
                         if(FAST_ACT) {
                             // relu / linear / leaky / relie: no transcendental, same predicates as nbl_act_apply
                             if(a.act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
@@ -368,7 +456,7 @@ void conv_igemm_kernel(const ConvArgs a) {
                         #pragma unroll
                         for(int j = 0; j < NT; j++) {
                             // an element without a residual keeps its value: adding a 0.0f placeholder would turn -0 into +0
-                            float t = (f < a.res_c && rok[j]) ? __fadd_rn(v[j], rv[e][j]) : v[j];
+                            float t = (f < a.res_c && rok[j]) ? __fadd_rn(v[j], rv[slot][e][j]) : v[j];
                             if(FAST_ACT) {
                                 if(a.post_act == NBL_ACT_RELU) t = t > 0.0f ? t : 0.0f;
                                 else if(a.post_act == NBL_ACT_LEAKY) t = t > 0.0f ? t : (float)(0.1 * (double)t);
@@ -414,23 +502,16 @@ void conv_igemm_kernel(const ConvArgs a) {
                 for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
         for(int kt = 0; kt < nkt; kt += 2) {
             // k-tile kt is in LDS buffer 0, kt+1 is in flight in stage 1
-#ifndef NBL_EXP_NO_GLOBAL
             ld_next(st0);
-#endif
             compute_tile(0);
             store_tile(st1, 1);
             __syncthreads();
             // k-tile kt+1 is in LDS buffer 1, kt+2 (possibly the next output tile's first) is in flight in stage 0
-#ifndef NBL_EXP_NO_GLOBAL
             ld_next(st1);
-#endif
             compute_tile(1);
             store_tile(st0, 0);
             __syncthreads();
         }
-#ifdef NBL_EXP_NO_EPILOGUE
-        if(acc[0][0][0] != 12345.678f) continue;
-#endif
         epilogue(tile);
     }
 }
@@ -545,7 +626,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false; p->persistent = false;
-    if(const char *e = getenv("NBL_CONV_PERSISTENT")) p->persistent = atoi(e) != 0; p->tuned_batch = 0; p->tuned_variant = -1;
+    p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL;
 
     // [F][K] -> [Kp][Mp], zero padded
@@ -626,6 +707,12 @@ static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev,
         fast_act = fast_act && (rs->post_act == NBL_ACT_RELU || rs->post_act == NBL_ACT_LINEAR ||
                                 rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE);
     }
+    const size_t out_bytes = (size_t)npix * p->F * sizeof(float);
+    const bool res_same_shape = rs && rs->c == p->F && rs->h == p->OH && rs->w == p->OW;
+    const bool sloped = p->act == NBL_ACT_LEAKY || p->act == NBL_ACT_RELIE ||
+                        (rs && (rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE));
+    a.short_epilogue = !(fast_act && out_bytes < (1ull << 32) && (!rs || res_same_shape) &&
+                         ((size_t)y_dev & 7) == 0 && (!rs || ((size_t)rs->res & 7) == 0)) ? 0 : sloped ? 2 : 1;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
     if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
        !p->force_scalar_gather)
