@@ -99,6 +99,16 @@ int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, 
 /* Pick the tile shape by hand (tests / tuning); variant < 0 restores the built-in choice.
  * nbl_conv2d_num_variants() says how many exist. */
 int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
+/* k-split of launches whose tile count leaves CUs idle in the last round: the tiles of that round are
+ * cut into slices along C*k*k, summed by a second small kernel in a fixed order (results do not depend
+ * on timing, but differ in the last bits from the unsplit sum order).  mode -1 (default): measured
+ * together with the tile shape on the first call at a batch size; 0: never; 1: wherever the built-in
+ * cost model says so.  No counterpart in the reference, whose GEMM is cuBLAS's choice
+ * (models/layers/convolutional_layer.cu:53-74). */
+int nbl_conv2d_plan_set_split(nbl_conv_plan *plan, int mode);
+/* Tile shape (index below nbl_conv2d_num_variants(), -1 before the first call) and number of k slices
+ * (1 = unsplit) of the plan's most recent launch. */
+int nbl_conv2d_plan_last_launch(const nbl_conv_plan *plan, int *variant, int *split_parts);
 int nbl_conv2d_num_variants(void);
 
 /* Replaces _im2col_ (common/utils.h:48, utils.cu:34-74; CPU twin utils.cc:81-119).  The convolution

@@ -44,6 +44,11 @@ struct ConvArgs {
     // output (and residual, when there is one and it has the output's shape) addressable with 32-bit byte
     // offsets and a cheap activation on both sides: full tiles may take the short epilogue
     int short_epilogue;   // 0: no, 1: relu/linear only, 2: leaky or relie somewhere
+    // split along k: blocks [0, whole_tiles) compute one whole tile each; after them every remaining tile
+    // is shared by `split` blocks, block part p accumulating its slice of the k-tiles and writing raw sums
+    // to ws[p][f][n - n_start]; conv_split_finish_kernel adds the parts and applies the epilogue
+    int whole_tiles, split, n_start, n_tail;
+    float *ws;
 };
 
 // Activation of the short epilogue, written as selects on uniform flags so that the epilogue stays one
@@ -137,11 +142,17 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     const int half = lane >> 5, l32 = lane & 31;
 
-    // Persistent blocks: block b works through output tiles b, b + gridDim.x, ... (m-tile fastest, so
-    // the blocks that share one pixel tile run next to each other).  The load side runs two k-tiles
-    // ahead of the MFMAs and simply crosses into the next output tile, so a tile's first loads overlap
-    // the previous tile's last MFMAs, and its epilogue stores drain while the next tile is multiplied.
-    const int total_tiles = a.tiles_m * a.tiles_n;
+    // which output tile, and which slice of its k-tiles, this block computes (all uniform)
+    const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
+    int tile = blockIdx.x, part = 0, kt_begin = 0, kt_end = nkt;
+    if(tile >= a.whole_tiles) {
+        const int u = tile - a.whole_tiles, pairs = nkt / 2;
+        tile = a.whole_tiles + u / a.split;
+        part = u % a.split;
+        kt_begin = 2 * (part * pairs / a.split);
+        kt_end = 2 * ((part + 1) * pairs / a.split);
+    }
+    const bool split_block = blockIdx.x >= a.whole_tiles;
 
     const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.x, a.x_bytes);
     const int ncol = tid % NCOLS;
@@ -151,17 +162,14 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int kgroup = VEC4 ? tid / NCOLS : __builtin_amdgcn_readfirstlane(tid / NCOLS);
     const int krow0 = VEC4 ? kgroup : kgroup * RB;
 
-    // ---- load side state: which output tile and k-tile the next global loads belong to ----
-    int ld_tile = blockIdx.x, ld_kt = 0, ld_m0 = 0;
+    // ---- load side state: the k-tile the next global loads belong to ----
+    int ld_kt = kt_begin;
+    const int ld_m0 = (tile % a.tiles_m) * BM;
     PixelCoord px;
-    unsigned xoff = 0;
-    const float *__restrict__ xpix = a.x;
-    auto ld_set_tile = [&](int tile) {
-        // past the block's last tile (pipeline tail) the loads repeat the last real tile; they are never used
-        const int t = tile < total_tiles ? tile : total_tiles - 1;
-        const int tm = t % a.tiles_m, tn = t / a.tiles_m;
-        ld_m0 = tm * BM;
-        const int n0 = tn * BN;
+    unsigned xoff;
+    const float *__restrict__ xpix;
+    {
+        const int n0 = (tile / a.tiles_m) * BN;
         // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past
         // the last pixel re-reads the last group (its results are never stored), a row past the last patch
         // row re-reads the last row and is zeroed when the tile is written to LDS.
@@ -170,7 +178,7 @@ void conv_igemm_kernel(const ConvArgs a) {
         // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
         xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
         xpix = a.x + (VEC4 ? px.xbase : 0);
-    };
+    }
 
     // Two register stages: the loads of k-tile t+2 are issued while k-tile t is multiplied and t+1 is
     // still in flight, so every global load has two k-tiles of MFMA time to arrive.
@@ -209,7 +217,8 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.b[r] = buf_load(xres, off);
             }
         }
-        const float *__restrict__ wtile = a.wp + (size_t)kt * BK * a.Mp + ld_m0;
+        // the pipeline runs two k-tiles past the block's last one: those loads repeat the last weight tile
+        const float *__restrict__ wtile = a.wp + (size_t)min(kt, nkt - 1) * BK * a.Mp + ld_m0;
         {
             const int row = tid / (BM / 4), col4 = tid % (BM / 4);
             if(A_VEC >= NTHREADS || tid < A_VEC)
@@ -222,16 +231,11 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.a1 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
         }
     };
-    const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
-    // issue the loads of the next k-tile in sequence and move the cursor (into the next output tile
-    // after the last k-tile of this one); the table entries of the k-tile after it follow
+    // issue the loads of the next k-tile; the table entries of the k-tile after it follow (the table ends
+    // in all-padding tiles for the pipeline's run past the last k-tile)
     auto ld_next = [&](Stage &st) {
         load_tile(st, ld_kt);
-        if(++ld_kt == nkt) {
-            ld_kt = 0;
-            ld_tile += gridDim.x;
-            ld_set_tile(ld_tile);
-        }
+        ++ld_kt;
         load_ktab(ld_kt);
     };
     auto store_tile = [&](const Stage &st, int buf) {
@@ -484,36 +488,84 @@ void conv_igemm_kernel(const ConvArgs a) {
         }
     };
 
-    // ---- pipeline start: k-tiles 0 and 1 of the block's first output tile ----
+    // Raw sums of a split block: ws[part][f][n - n_start], the lane's NT pixels as one vector where aligned.
+    auto store_partial = [&]() {
+        const int m0 = (tile % a.tiles_m) * BM, n0 = (tile / a.tiles_m) * BN;
+        const int nbase = n0 + wn * NT * 32 + l32 * NT;
+        if(nbase >= a.N) return;
+        float *__restrict__ wsp = a.ws + (size_t)part * a.F * a.n_tail + (nbase - a.n_start);
+        const bool vec_ok = NT == 2 && nbase + 1 < a.N && (a.n_tail & 1) == 0;
+        #pragma unroll
+        for(int r = 0; r < 16; r++) {
+            #pragma unroll
+            for(int i = 0; i < MT; i++) {
+                const int f = m0 + wm * MT * 32 + (8 * (r / 4) + 4 * half + r % 4) * MT + i;
+                if(f >= a.F) continue;
+                float *dst = wsp + (size_t)f * a.n_tail;
+                if(vec_ok) {
+                    *reinterpret_cast<float2*>(dst) = make_float2(acc[i][0][r], acc[i][NT - 1][r]);
+                } else {
+                    #pragma unroll
+                    for(int j = 0; j < NT; j++) if(nbase + j < a.N) dst[j] = acc[i][j][r];
+                }
+            }
+        }
+    };
+
+    // ---- pipeline start: the block's first two k-tiles ----
     st0.a0 = st0.a1 = st1.a0 = st1.a1 = make_float4(0.f, 0.f, 0.f, 0.f);
-    ld_set_tile(ld_tile);
-    load_ktab(0);
+    load_ktab(kt_begin);
     ld_next(st0);
     ld_next(st1);
     store_tile(st0, 0);
     __syncthreads();
 
-    for(int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    #pragma unroll
+    for(int i = 0; i < MT; i++)
         #pragma unroll
-        for(int i = 0; i < MT; i++)
+        for(int j = 0; j < NT; j++)
             #pragma unroll
-            for(int j = 0; j < NT; j++)
-                #pragma unroll
-                for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
-        for(int kt = 0; kt < nkt; kt += 2) {
-            // k-tile kt is in LDS buffer 0, kt+1 is in flight in stage 1
-            ld_next(st0);
-            compute_tile(0);
-            store_tile(st1, 1);
-            __syncthreads();
-            // k-tile kt+1 is in LDS buffer 1, kt+2 (possibly the next output tile's first) is in flight in stage 0
-            ld_next(st1);
-            compute_tile(1);
-            store_tile(st0, 0);
-            __syncthreads();
-        }
-        epilogue(tile);
+            for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    for(int kt = kt_begin; kt < kt_end - 2; kt += 2) {
+        // k-tile kt is in LDS buffer 0, kt+1 is in flight in stage 1
+        ld_next(st0);
+        compute_tile(0);
+        store_tile(st1, 1);
+        __syncthreads();
+        // k-tile kt+1 is in LDS buffer 1, kt+2 is in flight in stage 0
+        ld_next(st1);
+        compute_tile(1);
+        store_tile(st0, 0);
+        __syncthreads();
     }
+    // last pair: nothing left to load
+    compute_tile(0);
+    store_tile(st1, 1);
+    __syncthreads();
+    compute_tile(1);
+    if(split_block) store_partial();
+    else epilogue(tile);
+}
+
+// Second half of a k-split convolution: adds the parts in order and applies the epilogue the whole-tile
+// blocks apply themselves.  One thread per (filter, pixel column) of the split region.
+__global__ void conv_split_finish_kernel(const ConvArgs a) {
+    const int nloc = blockIdx.x * blockDim.x + threadIdx.x;
+    const int f = blockIdx.y;
+    if(nloc >= a.n_tail) return;
+    const size_t part_elems = (size_t)a.F * a.n_tail, at = (size_t)f * a.n_tail + nloc;
+    float t = a.ws[at];
+    for(int p = 1; p < a.split; p++) t = __fadd_rn(t, a.ws[p * part_elems + at]);
+    t = nbl_act_apply(a.act, __builtin_fmaf(t, a.g[f], a.b[f]));
+    const int n = a.n_start + nloc;
+    const int b = n / a.OHW, pix = n - b * a.OHW;
+    if(a.res && f < a.res_c) {
+        const int h = pix / a.OW, w = pix - h * a.OW;
+        if(h < a.res_box_h && w < a.res_box_w)
+            t = __fadd_rn(t, a.res[((size_t)b * a.res_c + f) * a.res_hw + h * a.res_stride * a.res_w + w * a.res_stride]);
+    }
+    if(a.res) t = nbl_act_apply(a.post_act, t);
+    a.y[((size_t)b * a.F + f) * a.OHW + pix] = t;
 }
 
 __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restrict__ ktab, float *__restrict__ col,
@@ -573,7 +625,10 @@ struct nbl_conv_plan {
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
     bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
-    bool persistent;            // blocks loop over several output tiles instead of taking exactly one (off: measured slower)
+    int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so
+    bool tuned_split;
+    float *ws_dev; size_t ws_bytes;   // partial sums of split launches (grown on demand)
+    int last_variant, last_split;     // what the most recent launch used
 };
 
 namespace {
@@ -594,6 +649,35 @@ int choose_variant(const nbl_conv_plan *p, unsigned N, int num_cu) {
         if(cost < best_cost) { best_cost = cost; best = v; }
     }
     return best;
+}
+
+// Which tiles of a launch are split along k, and into how many parts.  Blocks are dealt to CUs round
+// robin, so a launch takes as long as the CU with the most tiles: ceil(tiles / CUs) tile times, however
+// few tiles the last round holds.  The tiles of that last round (whole pixel-tile columns, so that the
+// split region is one range of pixel columns) are cut into `split` k-slices each so that they spread
+// over the idle CUs; the price is writing and re-reading the partial sums and one more small launch.
+struct SplitPlan { int whole_tiles, split; };
+
+SplitPlan plan_split(int tiles_m, int tiles_n, int bm, int bn, unsigned Kp, unsigned F, unsigned N, int num_cu) {
+    const int tiles = tiles_m * tiles_n, pairs = (int)(Kp / (2 * CONV_BK));
+    SplitPlan none = { tiles, 1 };
+    int whole = tiles / num_cu * num_cu;
+    whole -= whole % tiles_m;
+    const int left = tiles - whole;
+    if(left == 0 || pairs < 2) return none;
+    const double tile_us = 2.0 * bm * bn * Kp / (100e12 / num_cu) * 1e6;     // one CU, one tile, at a realistic rate
+    double best_us = std::ceil((double)left / num_cu) * tile_us;
+    int best = 1;
+    const size_t n_tail = N - (size_t)(whole / tiles_m) * bn;
+    for(int g = 2; g <= 8 && g <= pairs; g++) {
+        const size_t ws_bytes = (size_t)g * F * n_tail * sizeof(float);
+        if(ws_bytes > ((size_t)1 << 30)) break;
+        const double us = std::ceil((double)left * g / num_cu) / g * tile_us + 2.0 * ws_bytes / 4e12 * 1e6 + 5.0;
+        if(us < best_us) { best_us = us; best = g; }
+    }
+    if(best == 1) return none;
+    SplitPlan sp = { whole, best };
+    return sp;
 }
 
 }  // namespace
@@ -625,7 +709,8 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->K = C * ksize * ksize;
     p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
-    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false; p->persistent = false;
+    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false;
+    p->split_mode = -1; p->tuned_split = false; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL;
 
@@ -656,6 +741,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
 int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->wp_dev); nbl_free(ctx, p->ktab_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev);
+    nbl_free(ctx, p->ws_dev);
     delete p;
     return NBL_OK;
 }
@@ -674,10 +760,24 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
     return NBL_OK;
 }
 
+int nbl_conv2d_plan_set_split(nbl_conv_plan *p, int mode) {
+    if(!p || mode < -1 || mode > 1) return NBL_EINVAL;
+    p->split_mode = mode;
+    p->tuned_batch = 0;     // the next call searches again under the new rule
+    return NBL_OK;
+}
+
+int nbl_conv2d_plan_last_launch(const nbl_conv_plan *p, int *variant, int *split_parts) {
+    if(!p) return NBL_EINVAL;
+    if(variant) *variant = p->last_variant;
+    if(split_parts) *split_parts = p->last_split;
+    return NBL_OK;
+}
+
 struct ConvResidual { const float *res; unsigned c, h, w; int post_act; };
 
-static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v,
-                       const ConvResidual *rs) {
+static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v,
+                       bool split, const ConvResidual *rs) {
     const size_t in_elems = (size_t)B * p->C * p->H * p->W;
     const size_t npix = (size_t)B * p->OH * p->OW;
     const Variant &var = VARIANTS[v];
@@ -717,17 +817,34 @@ static int conv_launch(nbl_ctx *ctx, const nbl_conv_plan *p, const float *x_dev,
     if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
        !p->force_scalar_gather)
         gather = GATHER_1X1_VEC4;
-    // persistent grid: as many blocks as stay resident (by registers and LDS), each looping over its tiles;
-    // the count is rounded so that every block gets the same number of tiles where possible
+    a.whole_tiles = (int)blocks; a.split = 1; a.n_start = 0; a.n_tail = 0; a.ws = NULL;
     size_t grid = blocks;
-    const size_t resident = (size_t)ctx->num_cu * var.blocks_per_cu;
-    if(p->persistent && grid > resident) {
-        const size_t per_block = nbl_div_up_sz(blocks, resident);
-        grid = nbl_div_up_sz(blocks, per_block);
+    if(split && p->F <= 65535) {      // the finishing kernel's grid has one row per filter
+        const SplitPlan sp = plan_split(a.tiles_m, a.tiles_n, var.bm, var.bn, p->Kp, p->F, (unsigned)npix, ctx->num_cu);
+        if(sp.split > 1) {
+            a.whole_tiles = sp.whole_tiles; a.split = sp.split;
+            a.n_start = sp.whole_tiles / a.tiles_m * var.bn;
+            a.n_tail = (int)npix - a.n_start;
+            const size_t need = (size_t)sp.split * p->F * a.n_tail * sizeof(float);
+            if(need > p->ws_bytes) {
+                int rc = nbl_free(ctx, p->ws_dev);      // waits for launches that may still use it
+                p->ws_dev = NULL; p->ws_bytes = 0;
+                if(rc != NBL_OK || (rc = nbl_malloc(ctx, (void**)&p->ws_dev, need)) != NBL_OK) return rc;
+                p->ws_bytes = need;
+            }
+            a.ws = p->ws_dev;
+            grid = (size_t)sp.whole_tiles + (blocks - sp.whole_tiles) * sp.split;
+        }
     }
     hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)grid), dim3(var.threads), 0,
                        ctx->stream, a);
     NBL_LAUNCH_CHECK(ctx, "conv_igemm_kernel");
+    p->last_variant = v; p->last_split = a.split;
+    if(a.split > 1) {
+        hipLaunchKernelGGL(conv_split_finish_kernel, dim3(nbl_div_up((unsigned)a.n_tail, 256), p->F), dim3(256), 0,
+                           ctx->stream, a);
+        NBL_LAUNCH_CHECK(ctx, "conv_split_finish_kernel");
+    }
     return NBL_OK;
 }
 
@@ -741,20 +858,30 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
     hipError_t err = hipEventCreate(&e1);
     if(err != hipSuccess) { (void)hipEventDestroy(e0); return nbl_fail(ctx, NBL_EHIP, "hipEventCreate: %s", hipGetErrorString(err)); }
     int best = choose_variant(p, B * p->OH * p->OW, ctx->num_cu), rc = NBL_OK;
+    bool best_split = false;
     float best_ms = 1e30f;
     for(int v = 0; v < NUM_VARIANTS && rc == NBL_OK; v++) {
         if(nbl_div_up(p->F, VARIANTS[v].bm) * VARIANTS[v].bm > p->Mp) continue;
-        float ms = 0.0f;
-        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, rs)) != NBL_OK) break;
-        if(hipEventRecord(e0, ctx->stream) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed"); break; }
-        if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, rs)) != NBL_OK) break;
-        if(hipEventRecord(e1, ctx->stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
-           hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "event timing failed"); break; }
-        if(ms < best_ms) { best_ms = ms; best = v; }
+        for(int split = 0; split < 2 && rc == NBL_OK; split++) {
+            if(split != 0 && p->split_mode == 0) continue;
+            if(split == 0 && p->split_mode == 1) continue;
+            if(split != 0) {    // nothing to measure where the model splits nothing
+                const SplitPlan sp = plan_split(nbl_div_up(p->F, VARIANTS[v].bm), nbl_div_up(B * p->OH * p->OW, VARIANTS[v].bn),
+                                                VARIANTS[v].bm, VARIANTS[v].bn, p->Kp, p->F, B * p->OH * p->OW, ctx->num_cu);
+                if(sp.split <= 1 && p->split_mode != 1) continue;
+            }
+            float ms = 0.0f;
+            if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, split != 0, rs)) != NBL_OK) break;
+            if(hipEventRecord(e0, ctx->stream) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed"); break; }
+            if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, split != 0, rs)) != NBL_OK) break;
+            if(hipEventRecord(e1, ctx->stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+               hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "event timing failed"); break; }
+            if(ms < best_ms) { best_ms = ms; best = v; best_split = split != 0; }
+        }
     }
     (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
     if(rc != NBL_OK) return rc;
-    p->tuned_batch = B; p->tuned_variant = best;
+    p->tuned_batch = B; p->tuned_variant = best; p->tuned_split = best_split;
     return NBL_OK;
 }
 
@@ -766,15 +893,17 @@ static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_
     if(in_elems >= (1ull << 29) || out_elems >= (1ull << 31) || npix >= (1ull << 31) - 512)
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: inputs of 2^29 elements (2 GiB) or more are not supported");
     int v = p->variant;
+    bool split = p->split_mode == 1;
     if(v < 0) {
         if(p->tuned_batch != B) {
             // the search overwrites y with correct results several times; tiny problems are not worth it
-            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); }
+            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); p->tuned_split = p->split_mode == 1; }
             else { int rc = conv_tune(ctx, p, x_dev, y_dev, B, rs); if(rc != NBL_OK) return rc; }
         }
         v = p->tuned_variant;
+        split = p->tuned_split;
     }
-    return conv_launch(ctx, p, x_dev, y_dev, B, v, rs);
+    return conv_launch(ctx, p, x_dev, y_dev, B, v, split, rs);
 }
 
 int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {

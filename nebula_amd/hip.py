@@ -41,6 +41,8 @@ SIGNATURES = {
     "nbl_conv2d_plan_destroy": (C.c_int, [_vp, _vp]),
     "nbl_conv2d_plan_info": (C.c_int, [_vp, C.POINTER(_u), C.POINTER(_u), C.POINTER(C.c_double)]),
     "nbl_conv2d_plan_set_variant": (C.c_int, [_vp, C.c_int]),
+    "nbl_conv2d_plan_set_split": (C.c_int, [_vp, C.c_int]),
+    "nbl_conv2d_plan_last_launch": (C.c_int, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "nbl_conv2d_num_variants": (C.c_int, []),
     "nbl_im2col": (C.c_int, [_vp, _vp, _u, _u, _u, _u, _u, _u, _vp]),
     "nbl_fc_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, C.c_int, C.POINTER(_vp)]),
@@ -280,6 +282,16 @@ class ConvPlan:
 
     def set_variant(self, v):
         self.ctx.check(lib().nbl_conv2d_plan_set_variant(self.p, v))
+
+    def last_launch(self):
+        """(tile shape index, k slices) of the most recent launch."""
+        v, g = C.c_int(), C.c_int()
+        self.ctx.check(lib().nbl_conv2d_plan_last_launch(self.p, C.byref(v), C.byref(g)))
+        return v.value, g.value
+
+    def set_split(self, mode):
+        """-1: measured on first use, 0: never split along k, 1: split wherever the cost model says so."""
+        self.ctx.check(lib().nbl_conv2d_plan_set_split(self.p, mode))
 
     def __call__(self, x, out=None):
         B = x.shape[0]

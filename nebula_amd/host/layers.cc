@@ -154,6 +154,8 @@ void convolutional_layer_t::pack() {
                               input_channel, input_height, input_width, num_filters,
                               filter_size, stride, padding, (int)activation_type, &plan),
               "nbl_conv2d_pack");
+    if(network->conv_split >= 0)
+        nbl_check(network->ctx, nbl_conv2d_plan_set_split(plan, network->conv_split ? 1 : 0), "nbl_conv2d_plan_set_split");
 }
 
 bool convolutional_layer_t::fuse_with(shortcut_layer_t *m_shortcut) {

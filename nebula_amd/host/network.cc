@@ -22,7 +22,7 @@ network_t::network_t() :
     run_type(UNDEFINED_RUN), num_threads(1),
     learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
     input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
-    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), conv_split(-1),
     input_layer(NULL), output_layer(NULL), num_layers(0) {}
 
 network_t::~network_t() {}
@@ -117,6 +117,7 @@ void inference_net_t::build(config_t &config) {
             sc.get_setting("channels", &input_channel);
             sc.get_setting("batch", &batch_size);
             sc.get_setting("fuse_shortcut", &fuse_shortcut);
+            if(sc.exists("conv_split")) { unsigned v = 0; sc.get_setting("conv_split", &v); conv_split = v ? 1 : 0; }
             if(batch_override) batch_size = batch_override;
             input_size = input_height * input_width * input_channel;
             if(sc.exists("time_steps")) {

@@ -47,6 +47,10 @@ public:
     float *input_data_dev;              // device input [batch_size][input_size]
 
     nbl_ctx *ctx;                       // takes the place of cublas_handle / cudnn_handle
+    // [net] key `conv_split` (a key the reference ignores): 0 = convolutions never split their sum over
+    // the patch rows between blocks, 1 = wherever the cost model says so; absent = measured per layer on
+    // first use.  With 0 a convolution's result does not depend on the tile shape the search picks.
+    int conv_split;
 
     // Opens the headerless fp32 .wgh stream and lets every layer read its fields in cfg order
     // (models/networks/network.cc:99-122).

@@ -87,6 +87,63 @@ def test_conv_matches_oracle(ctx, case):
         assert rel(got, want) <= TOL, (case, v, rel(got, want))
 
 
+
+SPLIT = [
+    # B, C, H, W, F, k, s, p, bn, act, residual (None | "same" | "narrow"), post_act
+    (4, 64, 14, 14, 64, 3, 1, 1, True, "relu", None, "linear"),
+    (2, 96, 7, 7, 130, 3, 1, 1, False, "linear", "same", "relu"),       # odd plane, ragged F, fused shortcut
+    (3, 128, 10, 10, 40, 1, 1, 0, True, "leaky", "narrow", "leaky"),    # 1x1 vector gather, fewer residual channels
+    (1, 48, 9, 13, 24, 5, 2, 2, True, "logistic", None, "linear"),      # odd pixel count, exp-based activation
+    (5, 32, 12, 12, 256, 3, 1, 1, False, "relu", "same", "linear"),     # several filter tiles per pixel tile
+]
+
+
+@pytest.mark.parametrize("case", SPLIT)
+def test_conv_k_split_matches_oracle_and_unsplit(ctx, case):
+    """A launch split along the patch rows sums in another order: within tolerance of the oracle and of the
+    unsplit launch, for every tile shape, with and without the fused shortcut."""
+    from nebula_amd import hip
+    announce("conv split", case)
+    B, Cc, H, W, F, k, s, p, bn, act, residual, post = case
+    rng = np.random.default_rng(abs(hash(case[:8])) % (2 ** 31))
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    w = (rng.standard_normal((F, Cc, k, k)) * np.sqrt(2.0 / (Cc * k * k))).astype(np.float32)
+    bias = (rng.standard_normal(F) * 0.1).astype(np.float32)
+    bnp = None
+    if bn:
+        bnp = (rng.uniform(0.8, 1.2, F).astype(np.float32), (rng.standard_normal(F) * 0.1).astype(np.float32),
+               rng.uniform(0.5, 1.5, F).astype(np.float32))
+    want = ob.conv_forward(x, w, bias, bnp, s, p, act)
+    OH, OW = want.shape[2:]
+    conn = None
+    if residual:
+        conn = rng.standard_normal((B, F if residual == "same" else max(1, F // 3), OH, OW)).astype(np.float32)
+        want = ob.shortcut_forward(want, conn, post)
+    plan = ctx.conv_pack(w, bias, bnp, H=H, W=W, stride=s, pad=p, act=act)
+    dx = ctx.array(x)
+    dconn = ctx.array(conn) if conn is not None else None
+    run = (lambda: plan.with_shortcut(dx, dconn, post).numpy()) if residual else (lambda: plan(dx).numpy())
+    split_seen = 0
+    for v in range(hip.lib().nbl_conv2d_num_variants()):
+        plan.set_variant(v)
+        plan.set_split(0)
+        unsplit = run()
+        assert plan.last_launch() == (v, 1)
+        plan.set_split(1)
+        announce("conv split variant", v)
+        got = run()
+        split_seen += plan.last_launch()[1] > 1
+        assert rel(got, want) <= TOL, (case, v, rel(got, want))
+        assert rel(got, unsplit) <= 1e-5, (case, v, rel(got, unsplit))
+        again = run()
+        np.testing.assert_array_equal(bits(got), bits(again))           # fixed summation order
+    assert split_seen >= 3, "the cost model was expected to split most tile shapes of %r" % (case,)
+    plan.set_variant(-1)
+    plan.set_split(-1)
+    got = run()
+    assert rel(got, want) <= TOL
+
+
 def test_conv_relu_mask_matches_on_clear_margins(ctx):
     # outputs further than the tolerance from zero must land on the same side of the ReLU
     announce("conv relu mask")
