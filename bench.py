@@ -94,12 +94,33 @@ def cpu_baseline(cfg_fn, specs_weights, xdist, sample_batch, is_lstm, rng):
     return sample_batch / dt, cores, dt, ("OpenBLAS (scipy bundle)" if blas else "reference-style threaded GEMM"), x, outs
 
 
+def copy_calibration(args):
+    """K launches of the library's copy kernel over 256 MiB: reads 256 MiB and writes 256 MiB per launch."""
+    from nebula_amd import hip
+    ctx = hip.Ctx(0)
+    n = 64 << 20
+    src, dst = ctx.array(np.ones(n, np.float32)), ctx.empty((n,))
+    for _ in range(args.warmup):
+        ctx.copy(dst, src)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        ctx.copy(dst, src)
+    ms = ctx.timer_stop() / args.steps
+    print(json.dumps({"metric": "copy kernel GB/s (read+write)", "value": round(2 * 4 * n / ms / 1e6, 1), "unit": "GB/s",
+                      "bytes_read_per_launch": 4 * n, "bytes_written_per_launch": 4 * n, "steps": args.steps,
+                      "ms_per_launch": round(ms, 4)}), flush=True)
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1"])
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy"],
+                    help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
+                         "counters are calibrated against")
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -107,6 +128,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every layer is batch-parallel with no exchange; "
                  "more GPUs would each take batch/N images). Re-run with --gpus 1.")
+
+    if args.workload == "copy":
+        return copy_calibration(args)
 
     from nebula_amd.net import Network
 

@@ -64,6 +64,10 @@ int nbl_free(nbl_ctx *ctx, void *dev_ptr);
 int nbl_h2d(nbl_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);   /* returns after the copy */
 int nbl_d2h(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);   /* returns after the copy */
 int nbl_fill_zero(nbl_ctx *ctx, void *dst_dev, size_t bytes);                   /* a fill kernel, capturable */
+/* Device-to-device copy as a kernel on the context's stream (capturable; ranges must not overlap; both
+ * pointers 16-byte aligned).  Replaces the reference's cudaMemcpy(..., cudaMemcpyDeviceToDevice) between
+ * layer buffers (models/layers/lstm_layer.cu:41-55, models/layers/connected_layer.cu:244,282). */
+int nbl_copy_d2d(nbl_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 int nbl_sync(nbl_ctx *ctx);
 
 /* ---- convolution -------------------------------------------------------------------------------
@@ -100,8 +104,10 @@ int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, 
  * nbl_conv2d_num_variants() says how many exist. */
 int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
 /* k-split of launches whose tile count leaves CUs idle in the last round: the tiles of that round are
- * cut into slices along C*k*k, summed by a second small kernel in a fixed order (results do not depend
- * on timing, but differ in the last bits from the unsplit sum order).  mode -1 (default): measured
+ * cut into slices along C*k*k, one block each, and a second small kernel adds the slices in slice order
+ * and applies the epilogue (the result does not depend on timing, but it differs in the last bits from
+ * the unsplit sum order).  A plan keeps the scratch memory for this, so one plan must not run on two
+ * streams at once.  mode -1 (default): measured
  * together with the tile shape on the first call at a batch size; 0: never; 1: wherever the built-in
  * cost model says so.  No counterpart in the reference, whose GEMM is cuBLAS's choice
  * (models/layers/convolutional_layer.cu:53-74). */

@@ -548,24 +548,37 @@ void conv_igemm_kernel(const ConvArgs a) {
 }
 
 // Second half of a k-split convolution: adds the parts in order and applies the epilogue the whole-tile
-// blocks apply themselves.  One thread per (filter, pixel column) of the split region.
+// blocks apply themselves.  One thread per filter and VEC adjacent pixel columns of the split region;
+// VEC = 4 needs OH*OW and the region's width to be multiples of 4, so that a thread's pixels are one
+// aligned vector of one output plane.
+template<int VEC>
 __global__ void conv_split_finish_kernel(const ConvArgs a) {
-    const int nloc = blockIdx.x * blockDim.x + threadIdx.x;
+    typedef float __attribute__((ext_vector_type(VEC))) vec;
+    const int nloc = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     const int f = blockIdx.y;
     if(nloc >= a.n_tail) return;
     const size_t part_elems = (size_t)a.F * a.n_tail, at = (size_t)f * a.n_tail + nloc;
-    float t = a.ws[at];
-    for(int p = 1; p < a.split; p++) t = __fadd_rn(t, a.ws[p * part_elems + at]);
-    t = nbl_act_apply(a.act, __builtin_fmaf(t, a.g[f], a.b[f]));
+    vec t = *reinterpret_cast<const vec*>(a.ws + at);
+    for(int p = 1; p < a.split; p++) {
+        const vec u = *reinterpret_cast<const vec*>(a.ws + p * part_elems + at);
+        #pragma unroll
+        for(int e = 0; e < VEC; e++) t[e] = __fadd_rn(t[e], u[e]);
+    }
+    const float g = a.g[f], bias = a.b[f];
     const int n = a.n_start + nloc;
     const int b = n / a.OHW, pix = n - b * a.OHW;
-    if(a.res && f < a.res_c) {
-        const int h = pix / a.OW, w = pix - h * a.OW;
-        if(h < a.res_box_h && w < a.res_box_w)
-            t = __fadd_rn(t, a.res[((size_t)b * a.res_c + f) * a.res_hw + h * a.res_stride * a.res_w + w * a.res_stride]);
+    #pragma unroll
+    for(int e = 0; e < VEC; e++) {
+        float v = nbl_act_apply(a.act, __builtin_fmaf(t[e], g, bias));
+        if(a.res) {
+            const int h = (pix + e) / a.OW, w = (pix + e) - h * a.OW;
+            if(f < a.res_c && h < a.res_box_h && w < a.res_box_w)
+                v = __fadd_rn(v, a.res[((size_t)b * a.res_c + f) * a.res_hw + h * a.res_stride * a.res_w + w * a.res_stride]);
+            v = nbl_act_apply(a.post_act, v);
+        }
+        t[e] = v;
     }
-    if(a.res) t = nbl_act_apply(a.post_act, t);
-    a.y[((size_t)b * a.F + f) * a.OHW + pix] = t;
+    *reinterpret_cast<vec*>(a.y + ((size_t)b * a.F + f) * a.OHW + pix) = t;
 }
 
 __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restrict__ ktab, float *__restrict__ col,
@@ -841,8 +854,12 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     NBL_LAUNCH_CHECK(ctx, "conv_igemm_kernel");
     p->last_variant = v; p->last_split = a.split;
     if(a.split > 1) {
-        hipLaunchKernelGGL(conv_split_finish_kernel, dim3(nbl_div_up((unsigned)a.n_tail, 256), p->F), dim3(256), 0,
-                           ctx->stream, a);
+        if(a.OHW % 4 == 0 && a.n_tail % 4 == 0 && ((size_t)y_dev & 15) == 0)
+            hipLaunchKernelGGL(conv_split_finish_kernel<4>, dim3(nbl_div_up((unsigned)a.n_tail / 4, 256), p->F), dim3(256), 0,
+                               ctx->stream, a);
+        else
+            hipLaunchKernelGGL(conv_split_finish_kernel<1>, dim3(nbl_div_up((unsigned)a.n_tail, 256), p->F), dim3(256), 0,
+                               ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "conv_split_finish_kernel");
     }
     return NBL_OK;

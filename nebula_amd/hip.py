@@ -33,6 +33,7 @@ SIGNATURES = {
     "nbl_h2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_d2h": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "nbl_copy_d2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_sync": (C.c_int, [_vp]),
     "nbl_conv2d_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, _u, _u, _u, _u, _u, C.c_int,
                                   C.POINTER(_vp)]),
@@ -181,6 +182,12 @@ class Ctx:
 
     def sync(self):
         self.check(lib().nbl_sync(self.h))
+
+    def copy(self, dst, src, nbytes=None):
+        """Device-to-device copy kernel between two DeviceArrays."""
+        n = src.nbytes if nbytes is None else nbytes
+        assert n <= dst.nbytes and n <= src.nbytes
+        self.check(lib().nbl_copy_d2d(self.h, dst.ptr, src.ptr, n))
 
     def timer_start(self):
         self.check(lib().nbl_timer_start(self.h))

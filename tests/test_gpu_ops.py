@@ -176,6 +176,20 @@ def test_activation_kernels(ctx, name):
         np.testing.assert_array_equal(got > 0, x > 0)               # the mask itself
 
 
+def test_copy_d2d(ctx):
+    from nebula_amd import hip
+    announce("copy_d2d")
+    rng = np.random.default_rng(5)
+    for n in (1, 3, 4, 1023, 70001):
+        a = rng.standard_normal(n).astype(np.float32)
+        src, dst = ctx.array(a), ctx.array(np.zeros(n, np.float32))
+        ctx.copy(dst, src)
+        np.testing.assert_array_equal(bits(dst.numpy()), bits(a))
+    big = ctx.array(np.arange(64, dtype=np.float32))
+    rc = hip.lib().nbl_copy_d2d(ctx.h, big.ptr + 16, big.ptr, 64)
+    assert rc == -1 and b"overlap" in hip.lib().nbl_last_error(ctx.h)
+
+
 def test_activation_rejects_undefined(ctx):
     from nebula_amd import hip
     d = ctx.array(np.zeros(8, np.float32))
