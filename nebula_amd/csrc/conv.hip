@@ -49,6 +49,9 @@ struct ConvArgs {
     // to ws[p][f][n - n_start]; conv_split_finish_kernel adds the parts and applies the epilogue
     int whole_tiles, split, n_start, n_tail;
     float *ws;
+    // tap-major layers: one entry per k-tile, {byte offset of the tile's tap in channel c0's plane +
+    // c0*H*W*4, tap index i*ksize+j or -1 for an all-padding tile}
+    const int2 *ttab; int ksize; unsigned plane_bytes;
 };
 
 // Activation of the short epilogue, written as selects on uniform flags so that the epilogue stays one
@@ -111,10 +114,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float *p, unsi
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
 }
+// The range check looks at the per-lane offset only; the scalar offset is added afterwards.  A lane
+// whose offset is out of range therefore reads 0 whatever the scalar part is.
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byte_off, unsigned uniform_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, (int)uniform_off, 0));
+}
 // How a block gathers its slice of the patch matrix.
 enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
        GATHER_NOPAD = 1,    // padding = 0: every tap of a real pixel is inside the image
-       GATHER_1X1_VEC4 = 2  // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
+       GATHER_1X1_VEC4 = 2, // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
+       // Patch rows ordered (i, j, c) with C a multiple of the k-tile depth: a k-tile is 16 channels of ONE
+       // tap, so whether the tap is inside the image is decided once per pixel and k-tile (a bit of a mask
+       // computed at block start), and the 16 rows differ by a uniform plane offset that travels in the
+       // load's scalar offset.  Per gathered element no address or bounds arithmetic is left.
+       GATHER_TAP_MAJOR = 3
 };
 
 // OCC = blocks the register budget must leave room for on a CU (the persistent grid is sized with it)
@@ -125,7 +138,7 @@ void conv_igemm_kernel(const ConvArgs a) {
     constexpr int NTHREADS = 64 * WAVES_M * WAVES_N;
     constexpr int BM = MT * 32 * WAVES_M, BN = NT * 32 * WAVES_N;
     constexpr int LDA = BM + 32, LDB = BN + 32;        // rows k and k+1 land in different bank halves
-    constexpr bool VEC4 = GATHER == GATHER_1X1_VEC4;
+    constexpr bool VEC4 = GATHER == GATHER_1X1_VEC4, TAPM = GATHER == GATHER_TAP_MAJOR;
     constexpr int NCOLS = VEC4 ? BN / 4 : BN;          // column groups a k row is split into
     static_assert(NTHREADS % NCOLS == 0, "pixel columns must split evenly over threads");
     constexpr int KGROUPS = NTHREADS / NCOLS;          // thread groups along k
@@ -179,6 +192,13 @@ void conv_igemm_kernel(const ConvArgs a) {
         xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
         xpix = a.x + (VEC4 ? px.xbase : 0);
     }
+    unsigned tapmask = 0;       // tap-major: bit i*ksize+j set when that tap of this thread's pixel is inside the image
+    if(TAPM) {
+        int t = 0;
+        for(int i = 0; i < a.ksize; i++)
+            for(int j = 0; j < a.ksize; j++, t++)
+                if((unsigned)(px.ih0 + i) < (unsigned)a.H && (unsigned)(px.iw0 + j) < (unsigned)a.W) tapmask |= 1u << t;
+    }
 
     // Two register stages: the loads of k-tile t+2 are issued while k-tile t is multiplied and t+1 is
     // still in flight, so every global load has two k-tiles of MFMA time to arrive.
@@ -189,10 +209,12 @@ void conv_igemm_kernel(const ConvArgs a) {
         unsigned kvalid;
     };
     Stage st0, st1;
-    int2 ke[VEC4 ? 1 : RB];  // table entries of the next k-tile to gather
+    int2 ke[VEC4 || TAPM ? 1 : RB];  // table entries of the next k-tile to gather (tap-major: the k-tile's one entry)
 
     auto load_ktab = [&](int kt) {
-        if(!VEC4) {
+        if(TAPM) {
+            ke[0] = a.ttab[kt];
+        } else if(!VEC4) {
             const int2 *__restrict__ tp = a.ktab + kt * BK + krow0;
             #pragma unroll
             for(int r = 0; r < RB; r++) ke[r] = tp[r];
@@ -208,6 +230,11 @@ void conv_igemm_kernel(const ConvArgs a) {
                 // 1x1: input plane = output plane
                 st.b4[r] = *reinterpret_cast<const float4*>(xpix + (size_t)min(k, a.K - 1) * a.OHW);
             }
+        } else if(TAPM) {
+            const bool inside = ke[0].y >= 0 && ((tapmask >> (ke[0].y & 31)) & 1u) != 0;
+            const unsigned off = inside ? xoff + (unsigned)ke[0].x : OOB_OFFSET;   // stays out of range when xoff is
+            #pragma unroll
+            for(int r = 0; r < RB; r++) st.b[r] = buf_load(xres, off, (unsigned)(krow0 + r) * a.plane_bytes);
         } else {
             #pragma unroll
             for(int r = 0; r < RB; r++) {
@@ -590,13 +617,15 @@ __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restric
     col[(size_t)kk * OHW + pix] = conv_gather(x, p, ktab[kk], H, W);
 }
 
-// One entry per kk = (c*k + i)*k + j (the row order of the reference's col matrix).
-std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, unsigned Kp) {
+// One entry per patch row.  Reference order: kk = (c*k + i)*k + j (the row order of the reference's col
+// matrix); tap-major order: kk = (i*k + j)*C + c.
+std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, unsigned Kp, bool tap_major = false) {
     std::vector<int2> tab(Kp);
     const unsigned K = C * k * k;
     for(unsigned kk = 0; kk < Kp; kk++) {
         if(kk < K) {
-            const unsigned j = kk % k, i = (kk / k) % k, c = kk / k / k;
+            const unsigned j = tap_major ? (kk / C) % k : kk % k, i = tap_major ? kk / C / k : (kk / k) % k,
+                           c = tap_major ? kk % C : kk / k / k;
             tab[kk].x = (int)(c * H * W + i * W + j);
             tab[kk].y = (int)((i << 16) | j);
         } else {
@@ -607,16 +636,34 @@ std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, uns
     return tab;
 }
 
+// Tap-major layers: one entry per k-tile (see ConvArgs::ttab).
+std::vector<int2> build_ttab(unsigned C, unsigned H, unsigned W, unsigned k, unsigned tiles) {
+    std::vector<int2> tab(tiles);
+    const unsigned K = C * k * k;
+    for(unsigned kt = 0; kt < tiles; kt++) {
+        const unsigned kk = kt * CONV_BK;
+        if(kk < K) {
+            const unsigned t = kk / C, c0 = kk % C, i = t / k, j = t % k;
+            tab[kt].x = (int)((c0 * H * W + i * W + j) * 4);
+            tab[kt].y = (int)t;
+        } else {
+            tab[kt].x = 0; tab[kt].y = -1;
+        }
+    }
+    return tab;
+}
+
 typedef void (*ConvKernel)(const ConvArgs);
 // kernel[gather mode][any activation ? 1 : 0]
-struct Variant { int bm, bn, threads, blocks_per_cu; ConvKernel kernel[3][2]; const char *name; };
+struct Variant { int bm, bn, threads, blocks_per_cu; ConvKernel kernel[4][2]; const char *name; };
 
 // blocks_per_cu: resident blocks per CU (register- and LDS-limited), the size of the persistent grid
 #define NBL_CONV_VARIANT(MT, NT, WM, WN, OCC, NAME) \
     { MT * 32 * WM, NT * 32 * WN, 64 * WM * WN, OCC, \
       { { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_PADDED, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_PADDED, false> }, \
         { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_NOPAD, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_NOPAD, false> }, \
-        { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, false> } }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_1X1_VEC4, false> }, \
+        { conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_TAP_MAJOR, true>, conv_igemm_kernel<MT, NT, WM, WN, OCC, GATHER_TAP_MAJOR, false> } }, \
       NAME }
 
 const Variant VARIANTS[] = {
@@ -635,6 +682,7 @@ struct nbl_conv_plan {
     unsigned C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp;
     int act; bool has_scale;
     float *wp_dev; int2 *ktab_dev; float *g_dev; float *b_dev;
+    bool tap_major; int2 *ttab_dev;   // patch rows in (i, j, c) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 32)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
     bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
@@ -725,19 +773,28 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false;
     p->split_mode = -1; p->tuned_split = false; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
-    p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL;
+    p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
+    p->tap_major = ksize > 1 && ksize * ksize <= 32 && C % CONV_BK == 0;
 
     // [F][K] -> [Kp][Mp], zero padded
     std::vector<float> wp((size_t)p->Kp * p->Mp, 0.0f);
+    const unsigned taps = ksize * ksize;
     for(unsigned f = 0; f < F; f++)
-        for(unsigned kk = 0; kk < p->K; kk++) wp[(size_t)kk * p->Mp + f] = weight_host[(size_t)f * p->K + kk];
+        for(unsigned kk = 0; kk < p->K; kk++) {
+            // kk = c*taps + t in the file; row t*C + c in a tap-major layer
+            const unsigned row = p->tap_major ? (kk % taps) * C + kk / taps : kk;
+            wp[(size_t)row * p->Mp + f] = weight_host[(size_t)f * p->K + kk];
+        }
     std::vector<float> g(p->Mp, 0.0f), b(p->Mp, 0.0f);
     nbl_fold_batchnorm(bias_host, scale_host, mean_host, var_host, F, g.data(), b.data());
-    std::vector<int2> tab = build_ktab(C, H, W, ksize, p->Kp + 4 * CONV_BK);   // + all-padding tiles read by the pipeline tail
+    std::vector<int2> tab = build_ktab(C, H, W, ksize, p->Kp + 4 * CONV_BK, p->tap_major);   // + all-padding tiles behind the last k-tile
+    std::vector<int2> ttab = build_ttab(C, H, W, ksize, p->Kp / CONV_BK + 4);
 
     int rc;
     if((rc = nbl_malloc(ctx, (void**)&p->wp_dev, wp.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->ktab_dev, tab.size() * sizeof(int2))) != NBL_OK ||
+       (rc = nbl_malloc(ctx, (void**)&p->ttab_dev, ttab.size() * sizeof(int2))) != NBL_OK ||
+       (rc = nbl_h2d(ctx, p->ttab_dev, ttab.data(), ttab.size() * sizeof(int2))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->g_dev, g.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->b_dev, b.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_h2d(ctx, p->wp_dev, wp.data(), wp.size() * sizeof(float))) != NBL_OK ||
@@ -753,6 +810,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
 
 int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
+    nbl_free(ctx, p->ttab_dev);
     nbl_free(ctx, p->wp_dev); nbl_free(ctx, p->ktab_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev);
     nbl_free(ctx, p->ws_dev);
     delete p;
@@ -826,7 +884,9 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
                         (rs && (rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE));
     a.short_epilogue = !(fast_act && out_bytes < (1ull << 32) && (!rs || res_same_shape) &&
                          ((size_t)y_dev & 7) == 0 && (!rs || ((size_t)rs->res & 7) == 0)) ? 0 : sloped ? 2 : 1;
+    a.ttab = p->ttab_dev; a.ksize = (int)p->k; a.plane_bytes = p->H * p->W * 4u;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
+    if(p->tap_major && !p->force_scalar_gather) gather = GATHER_TAP_MAJOR;
     if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
        !p->force_scalar_gather)
         gather = GATHER_1X1_VEC4;
