@@ -61,6 +61,10 @@ const char *nbl_last_error(nbl_ctx *ctx);
 void *nbl_ctx_stream(nbl_ctx *ctx);
 int nbl_malloc(nbl_ctx *ctx, void **dev_ptr, size_t bytes);
 int nbl_free(nbl_ctx *ctx, void *dev_ptr);
+/* Page-locked host memory: nbl_h2d / nbl_d2h to and from it skip the driver's staging copy.  The
+ * reference keeps its host-side layer outputs in plain new[] arrays (models/layers/softmax_layer.cc:34). */
+int nbl_malloc_host(nbl_ctx *ctx, void **host_ptr, size_t bytes);
+int nbl_free_host(nbl_ctx *ctx, void *host_ptr);
 int nbl_h2d(nbl_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);   /* returns after the copy */
 int nbl_d2h(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);   /* returns after the copy */
 int nbl_fill_zero(nbl_ctx *ctx, void *dst_dev, size_t bytes);                   /* a fill kernel, capturable */

@@ -112,6 +112,24 @@ int nbl_free(nbl_ctx *ctx, void *dev_ptr) {
     return NBL_OK;
 }
 
+int nbl_malloc_host(nbl_ctx *ctx, void **host_ptr, size_t bytes) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, host_ptr != NULL, "nbl_malloc_host: host_ptr is NULL");
+    *host_ptr = NULL;
+    if(bytes == 0) return NBL_OK;
+    NBL_HIP(ctx, hipSetDevice(ctx->device));
+    NBL_HIP(ctx, hipHostMalloc(host_ptr, bytes, hipHostMallocDefault));
+    return NBL_OK;
+}
+
+int nbl_free_host(nbl_ctx *ctx, void *host_ptr) {
+    if(!ctx) return NBL_EINVAL;
+    if(!host_ptr) return NBL_OK;
+    NBL_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    NBL_HIP(ctx, hipHostFree(host_ptr));
+    return NBL_OK;
+}
+
 int nbl_h2d(nbl_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
     if(!ctx) return NBL_EINVAL;
     if(bytes == 0) return NBL_OK;

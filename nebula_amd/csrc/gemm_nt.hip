@@ -286,7 +286,8 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     int S = 1;
     const int ktiles = nbl_div_up(K, GEMM_BK);
     if(ws) {
-        while(S < 16 && (size_t)gm * gn * S < 2u * ctx->num_cu && ktiles / (S * 2) >= 8) S *= 2;
+        // (a block's time is mostly its serial walk over k, so short chunks pay even at 2 k-tiles each)
+        while(S < 64 && (size_t)gm * gn * S < 2u * ctx->num_cu && ktiles / (S * 2) >= 2) S *= 2;
     }
     a.k_chunk = nbl_div_up(ktiles, S) * GEMM_BK;
     S = nbl_div_up(K, a.k_chunk);

@@ -1,5 +1,6 @@
 #include "layers.h"
 
+#include <algorithm>
 #include <cmath>
 #include <random>
 #include <stdexcept>
@@ -28,7 +29,7 @@ layer_t::layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_lay
     layer_type(m_layer_type), activation_type(UNDEFINED_ACTIVATION),
     input_height(1), input_width(1), input_channel(1), input_size(1),
     output_height(1), output_width(1), output_channel(1), output_size(0),
-    output_data(NULL), delta(NULL),
+    output_data(NULL), delta(NULL), output_data_pinned(false),
     padding(0), num_filters(1), filter_size(1), stride(1), group(1),
     prev_layer(m_prev_layer), next_layer(NULL),
     output_data_dev(NULL), delta_dev(NULL),
@@ -38,7 +39,8 @@ layer_t::layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_lay
 
 layer_t::~layer_t() {
     if(owns_output && output_data_dev && network->ctx) nbl_free(network->ctx, output_data_dev);
-    delete [] output_data;
+    if(output_data_pinned) nbl_free_host(network->ctx, output_data);
+    else delete [] output_data;
 }
 
 void layer_t::backward() { inference_only("backward()"); }
@@ -378,7 +380,14 @@ softmax_layer_t::~softmax_layer_t() {}
 void softmax_layer_t::init(section_config_t) {
     input_size = prev_layer ? prev_layer->output_size : network->input_size;
     output_size = input_size;
-    output_data = new float[(size_t)output_size * network->batch_size]();
+    const size_t count = (size_t)output_size * network->batch_size;
+    if(network->ctx) {      // page-locked, so the per-forward copy of the probabilities needs no staging
+        nbl_check(network->ctx, nbl_malloc_host(network->ctx, (void**)&output_data, count * sizeof(float)), "nbl_malloc_host(softmax)");
+        output_data_pinned = true;
+        std::fill(output_data, output_data + count, 0.0f);
+    } else {
+        output_data = new float[count]();
+    }
     alloc_output();
 }
 

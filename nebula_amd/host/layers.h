@@ -45,6 +45,7 @@ public:
     unsigned output_height, output_width, output_channel, output_size;
 
     float *output_data;        // host copy; only the softmax layer fills it (as the reference's GPU path)
+    bool output_data_pinned;            // output_data came from nbl_malloc_host
     float *delta;              // never allocated (training)
 
     unsigned padding, num_filters, filter_size, stride, group;
