@@ -48,6 +48,7 @@ struct ConvArgs {
     // is shared by `split` blocks, block part p accumulating its slice of the k-tiles and writing raw sums
     // to ws[p][f][n - n_start]; conv_split_finish_kernel adds the parts and applies the epilogue
     int whole_tiles, split, n_start, n_tail;
+    int units;     // whole_tiles + (tiles - whole_tiles) * split: work units of the launch
     float *ws;
     // tap-major layers: one entry per k-tile, {byte offset of the tile's tap in channel c0's plane +
     // c0*H*W*4, tap index i*ksize+j or -1 for an all-padding tile}
@@ -123,8 +124,8 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byt
 enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
        GATHER_NOPAD = 1,    // padding = 0: every tap of a real pixel is inside the image
        GATHER_1X1_VEC4 = 2, // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
-       // Patch rows ordered (i, j, c) with C a multiple of the k-tile depth: a k-tile is 16 channels of ONE
-       // tap, so whether the tap is inside the image is decided once per pixel and k-tile (a bit of a mask
+       // Patch rows ordered (c / 16, i, j, c % 16) with C a multiple of the k-tile depth: a k-tile is 16
+       // channels of ONE tap, so whether the tap is inside the image is decided once per pixel and k-tile (a bit of a mask
        // computed at block start), and the 16 rows differ by a uniform plane offset that travels in the
        // load's scalar offset.  Per gathered element no address or bounds arithmetic is left.
        GATHER_TAP_MAJOR = 3
@@ -157,7 +158,19 @@ void conv_igemm_kernel(const ConvArgs a) {
 
     // which output tile, and which slice of its k-tiles, this block computes (all uniform)
     const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
-    int tile = blockIdx.x, part = 0, kt_begin = 0, kt_end = nkt;
+    // Workgroups are dealt to the 8 XCDs round robin by index, and each XCD has its own L2.  The work
+    // units are therefore renumbered so that a run of tiles_m consecutive units (the filter tiles of one
+    // pixel tile, which read the same input) lands on one XCD, runs being dealt round robin in turn.
+    int tile;
+    {
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run = slot / (unsigned)a.tiles_m,
+                       within = slot - run * (unsigned)a.tiles_m;
+        const unsigned unit = (run * 8u + xcd) * (unsigned)a.tiles_m + within;
+        if(unit >= (unsigned)a.units) return;         // the grid is padded to whole rounds of runs
+        tile = (int)unit;
+    }
+    const int unit = tile;
+    int part = 0, kt_begin = 0, kt_end = nkt;
     if(tile >= a.whole_tiles) {
         const int u = tile - a.whole_tiles, pairs = nkt / 2;
         tile = a.whole_tiles + u / a.split;
@@ -165,7 +178,7 @@ void conv_igemm_kernel(const ConvArgs a) {
         kt_begin = 2 * (part * pairs / a.split);
         kt_end = 2 * ((part + 1) * pairs / a.split);
     }
-    const bool split_block = blockIdx.x >= a.whole_tiles;
+    const bool split_block = unit >= a.whole_tiles;
 
     const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.x, a.x_bytes);
     const int ncol = tid % NCOLS;
@@ -617,33 +630,39 @@ __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restric
     col[(size_t)kk * OHW + pix] = conv_gather(x, p, ktab[kk], H, W);
 }
 
-// One entry per patch row.  Reference order: kk = (c*k + i)*k + j (the row order of the reference's col
-// matrix); tap-major order: kk = (i*k + j)*C + c.
+// Row of the packed patch matrix that holds channel c, tap t = i*k + j.  Reference order (the row
+// order of the reference's col matrix): (c*k + i)*k + j.  Tap-major order: channels in groups of the
+// k-tile depth, within a group the taps, within a tap the group's channels, so that a k-tile is 16
+// channels of one tap and the k-tiles that follow revisit the same 16 input planes for the other taps
+// while they are still in cache.
+inline unsigned patch_row(unsigned c, unsigned t, unsigned taps, bool tap_major) {
+    return tap_major ? (c / CONV_BK) * (taps * CONV_BK) + t * CONV_BK + c % CONV_BK : c * taps + t;
+}
+
+// One entry per patch row, in packed order.
 std::vector<int2> build_ktab(unsigned C, unsigned H, unsigned W, unsigned k, unsigned Kp, bool tap_major = false) {
     std::vector<int2> tab(Kp);
-    const unsigned K = C * k * k;
     for(unsigned kk = 0; kk < Kp; kk++) {
-        if(kk < K) {
-            const unsigned j = tap_major ? (kk / C) % k : kk % k, i = tap_major ? kk / C / k : (kk / k) % k,
-                           c = tap_major ? kk % C : kk / k / k;
-            tab[kk].x = (int)(c * H * W + i * W + j);
-            tab[kk].y = (int)((i << 16) | j);
-        } else {
-            tab[kk].x = 0;
-            tab[kk].y = (int)0x80000000u | (KTAB_PAD_TAP << 16);   // sign bit: padding row
-        }
+        tab[kk].x = 0;
+        tab[kk].y = (int)0x80000000u | (KTAB_PAD_TAP << 16);   // sign bit: padding row
     }
+    for(unsigned c = 0; c < C; c++)
+        for(unsigned i = 0; i < k; i++)
+            for(unsigned j = 0; j < k; j++) {
+                const unsigned kk = patch_row(c, i * k + j, k * k, tap_major);
+                tab[kk].x = (int)(c * H * W + i * W + j);
+                tab[kk].y = (int)((i << 16) | j);
+            }
     return tab;
 }
 
 // Tap-major layers: one entry per k-tile (see ConvArgs::ttab).
 std::vector<int2> build_ttab(unsigned C, unsigned H, unsigned W, unsigned k, unsigned tiles) {
     std::vector<int2> tab(tiles);
-    const unsigned K = C * k * k;
+    const unsigned taps = k * k, K = C * taps;
     for(unsigned kt = 0; kt < tiles; kt++) {
-        const unsigned kk = kt * CONV_BK;
-        if(kk < K) {
-            const unsigned t = kk / C, c0 = kk % C, i = t / k, j = t % k;
+        if(kt * CONV_BK < K) {
+            const unsigned t = kt % taps, c0 = kt / taps * CONV_BK, i = t / k, j = t % k;
             tab[kt].x = (int)((c0 * H * W + i * W + j) * 4);
             tab[kt].y = (int)t;
         } else {
@@ -682,7 +701,7 @@ struct nbl_conv_plan {
     unsigned C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp;
     int act; bool has_scale;
     float *wp_dev; int2 *ktab_dev; float *g_dev; float *b_dev;
-    bool tap_major; int2 *ttab_dev;   // patch rows in (i, j, c) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 32)
+    bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 32)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
     bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
@@ -781,8 +800,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     const unsigned taps = ksize * ksize;
     for(unsigned f = 0; f < F; f++)
         for(unsigned kk = 0; kk < p->K; kk++) {
-            // kk = c*taps + t in the file; row t*C + c in a tap-major layer
-            const unsigned row = p->tap_major ? (kk % taps) * C + kk / taps : kk;
+            const unsigned row = patch_row(kk / taps, kk % taps, taps, p->tap_major);    // kk = c*taps + t in the file
             wp[(size_t)row * p->Mp + f] = weight_host[(size_t)f * p->K + kk];
         }
     std::vector<float> g(p->Mp, 0.0f), b(p->Mp, 0.0f);
@@ -909,6 +927,10 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
             grid = (size_t)sp.whole_tiles + (blocks - sp.whole_tiles) * sp.split;
         }
     }
+    a.units = (int)grid;
+    const size_t round = 8u * (size_t)a.tiles_m;
+    grid = nbl_div_up_sz(grid, round) * round;
+    if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)grid), dim3(var.threads), 0,
                        ctx->stream, a);
     NBL_LAUNCH_CHECK(ctx, "conv_igemm_kernel");
