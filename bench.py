@@ -25,6 +25,12 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 
+# HBM bytes per average launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over
+# this script (each counter scaled by what it reads for `--workload copy`, 256 MiB in and out per
+# launch): a recorded measurement, valid for the named workload and batch only.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("resnet50", 64): 168.7e6}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -113,14 +119,46 @@ def copy_calibration(args):
     ctx.close()
 
 
+def single_conv(args):
+    """One convolution layer (bias + ReLU epilogue) at batch --batch (default 64) through nbl_conv2d_fwd."""
+    from nebula_amd import hip
+    C_, H, W, F, k, st, pad = (int(v) for v in args.conv_shape.split(","))
+    B = args.batch or 64
+    ctx = hip.Ctx(0)
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((F, C_, k, k)) * np.sqrt(2.0 / (C_ * k * k))).astype(np.float32)
+    plan = ctx.conv_pack(w, np.zeros(F, np.float32), None, H=H, W=W, stride=st, pad=pad, act="relu")
+    plan.set_variant(args.conv_variant)
+    plan.set_split(args.conv_split)
+    x = ctx.array(rng.standard_normal((B, C_, H, W)).astype(np.float32))
+    y = ctx.empty((B, F, plan.OH, plan.OW))
+    for _ in range(args.warmup):
+        plan(x, out=y)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        plan(x, out=y)
+    ms = ctx.timer_stop() / args.steps
+    variant, parts = plan.last_launch()
+    flop = plan.flop_per_image * B
+    print(json.dumps({"metric": "conv layer TFLOP/s", "value": round(flop / ms / 1e9, 2), "unit": "TFLOP/s", "shape": args.conv_shape,
+                      "batch": B, "gemm": {"M": F, "N": B * plan.OH * plan.OW, "K": C_ * k * k}, "tile_variant": variant,
+                      "k_slices": parts, "ms_per_launch": round(ms, 4), "steps": args.steps}), flush=True)
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
-                         "counters are calibrated against")
+                         "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
+                         "for counter passes over a single kernel")
+    ap.add_argument("--conv-shape", default="512,28,28,256,1,1,0", help="C,H,W,F,k,stride,pad of --workload conv")
+    ap.add_argument("--conv-variant", type=int, default=-1, help="tile shape index of --workload conv (-1: searched)")
+    ap.add_argument("--conv-split", type=int, default=-1, help="k-split mode of --workload conv (-1 searched, 0 off, 1 model)")
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -131,6 +169,8 @@ def main():
 
     if args.workload == "copy":
         return copy_calibration(args)
+    if args.workload == "conv":
+        return single_conv(args)
 
     from nebula_amd.net import Network
 
@@ -177,6 +217,8 @@ def main():
     for k, ms in zip(kinds, layer_ms):
         by_kind[k] = by_kind.get(k, 0.0) + ms
     log("per-layer-kind ms:", {k: round(v, 3) for k, v in by_kind.items()})
+    algo_bytes = 0.0
+    fused = "fuse_shortcut=1" in cfg
     if is_lstm:
         # 2*B*(I+H)*4H per step per layer
         lstm_flop = sum(2.0 * net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])
@@ -191,9 +233,19 @@ def main():
         n_launch = len(conv)
         achieved = float(flops[conv].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
         dom_name = "conv_igemm_kernel"
+        # algorithmic bytes of the same launches: input + weights + output (+ the residual a fused shortcut reads)
+        for i in conv:
+            info = net.layer_info(i)
+            weights = net.layer_flop(i) / (2.0 * info["output_height"] * info["output_width"])
+            residual = info["output_size"] if i + 1 < len(kinds) and kinds[i + 1] == "shortcut_layer" and fused else 0
+            algo_bytes += 4.0 * (net.batch_size * (info["input_size"] + info["output_size"] + residual) + weights)
     roofline = {"bound": "mfma", "kernel": dom_name, "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, batch)),
                 "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4)}
+    if algo_bytes:
+        roofline["algorithmic_bytes_per_launch"] = round(algo_bytes / n_launch)
+        roofline["algorithmic_flop_per_launch"] = round(float(flops[conv].sum()) / n_launch)
 
     result = {
         "metric": "ResNet-50 fp32 fwd images/s (bs64, 1 GPU); conv GEMM % of fp32 MFMA peak" if args.workload == "resnet50"
