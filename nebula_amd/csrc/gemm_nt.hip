@@ -18,6 +18,7 @@
 #include "nbl_internal.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -40,6 +41,15 @@ struct GemmArgs {
     // sub_act), b = recurrent-side bias, act = sub_act; c [M][H] cell state (in place), C = h out [M][H]
     const float *gx; float *c; int H;
 };
+
+// Gate non-linearities of the LSTM cell in single precision (the layer's tolerance is 1e-4 relative;
+// expf is good to an ulp or two).  tanh follows the reference's (e^{2x} - 1) / (e^{2x} + 1) with the
+// argument clamped where that quotient has long rounded to +-1, so it cannot overflow.
+__device__ __forceinline__ float lstm_logistic(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float lstm_tanh(float x) {
+    const float e = expf(2.0f * fminf(fmaxf(x, -15.0f), 15.0f));
+    return (e - 1.0f) / (e + 1.0f);
+}
 
 __device__ __forceinline__ float4 load_row4(const float *__restrict__ base, int row, int rows, int ld,
                                             int k, int K, int vec_ok) {
@@ -165,17 +175,17 @@ void gemm_nt_kernel(const GemmArgs a) {
                         const int n = hb * 128 + gate * 32 + l32;
                         pre[gate] = nbl_act_apply(a.act, acc[i][gate % NT][r] + a.b[n]) + a.gx[(size_t)m * a.ldc + n];
                     }
-                    const float gi = nbl_act_apply(NBL_ACT_LOGISTIC, pre[0]);
-                    const float gf = nbl_act_apply(NBL_ACT_LOGISTIC, pre[1]);
-                    const float gg = nbl_act_apply(NBL_ACT_TANH, pre[2]);
-                    const float go = nbl_act_apply(NBL_ACT_LOGISTIC, pre[3]);
+                    const float gi = lstm_logistic(pre[0]);
+                    const float gf = lstm_logistic(pre[1]);
+                    const float gg = lstm_tanh(pre[2]);
+                    const float go = lstm_logistic(pre[3]);
                     // c_t = c_{t-1}*f + i*g with each product rounded, as the reference's separate passes do
                     const size_t e = (size_t)m * a.H + h;
                     const float ig = __fmul_rn(gi, gg);
                     const float cf = __fmul_rn(a.c[e], gf);
                     const float ct = __fadd_rn(cf, ig);
                     a.c[e] = ct;
-                    a.C[e] = __fmul_rn(nbl_act_apply(NBL_ACT_TANH, ct), go);
+                    a.C[e] = __fmul_rn(lstm_tanh(ct), go);
                 }
         }
         return;
@@ -217,6 +227,93 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__re
     y[e] = nbl_act_apply(act, v);
 }
 
+// One LSTM time step in one launch, for layers packed with gate interleave 8 (row of gate g, hidden unit
+// h: (h/8)*32 + g*8 + h%8), so that ONE 32x32 MFMA tile holds the four gate pre-activations of 8 hidden
+// units for 32 batch rows.  A step is latency, not throughput ([B x H].[H x 4H] is 3.4 us of MFMA time
+// on the whole chip), so the work is cut for many small independent pieces: a block owns one such
+// tile, its four waves each take a quarter of the k range and read their MFMA operands STRAIGHT from
+// global memory (each lane one 16-byte piece of its row per 8 k: lanes 0-31 supply k+0..3, lanes
+// 32-63 k+4..7 of both operands, which is a legal pairing), several loads in flight per lane and no
+// barrier until the four partial tiles meet in LDS.  Then each thread owns one (batch row, hidden
+// unit): sum of the four partial tiles for each gate, bias, input-side pre-activation, the cell update
+// (lstm_layer.cc:264-312, each product rounded on its own) and h_t written into y[t], which is the
+// next step's operand.  Needs H % 128 == 0 and 16-byte aligned rows.
+struct LstmStepArgs {
+    const float *hprev; const float *w; const float *gx; const float *bw; float *c; float *hout;
+    int B, H, Np, sub_act;
+};
+
+__global__ __launch_bounds__(256)
+void lstm_step_kernel(const LstmStepArgs a) {
+    constexpr int U = 4;                    // 8-wide k steps per batch of loads
+    __shared__ float red[4][32][33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int kw = a.H >> 2;                // k range of one wave
+    const int arow = min(m0 + r, a.B - 1);  // rows past the batch repeat the last one; their sums are dropped
+    const float *__restrict__ ap = a.hprev + (size_t)arow * a.H + wave * kw + half * 4;
+    const float *__restrict__ bp = a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4;
+    const int nb = kw / (8 * U);
+
+    float4 av[2][U], bv[2][U];
+    auto load = [&](int buf, int b) {
+        #pragma unroll
+        for(int u = 0; u < U; u++) {
+            av[buf][u] = *reinterpret_cast<const float4*>(ap + (b * U + u) * 8);
+            bv[buf][u] = *reinterpret_cast<const float4*>(bp + (b * U + u) * 8);
+        }
+    };
+    // two accumulators take turns: with one wave per SIMD nothing else hides the latency between two
+    // MFMAs on the same registers
+    floatx16 acc0, acc1;
+    #pragma unroll
+    for(int i = 0; i < 16; i++) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
+    auto compute = [&](int buf) {
+        #pragma unroll
+        for(int u = 0; u < U; u++) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[buf][u].x, bv[buf][u].x, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[buf][u].y, bv[buf][u].y, acc1, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[buf][u].z, bv[buf][u].z, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[buf][u].w, bv[buf][u].w, acc1, 0, 0, 0);
+        }
+    };
+    load(0, 0);
+    int b = 0;
+    for(; b + 2 <= nb; b += 2) {
+        load(1, b + 1);
+        compute(0);
+        if(b + 2 < nb) load(0, b + 2);
+        compute(1);
+    }
+    if(b < nb) compute(0);
+
+    // accumulator register i of a 32x32 tile: row 8*(i/4) + 4*(lane/32) + i%4 (batch), column lane%32 (gate column)
+    #pragma unroll
+    for(int i = 0; i < 16; i++) red[wave][8 * (i >> 2) + 4 * half + (i & 3)][r] = acc0[i] + acc1[i];
+    __syncthreads();
+    const int ml = tid >> 3, hh = tid & 7;
+    const int m = m0 + ml, h = blockIdx.x * 8 + hh;
+    if(m >= a.B) return;
+    float pre[4];
+    #pragma unroll
+    for(int gate = 0; gate < 4; gate++) {
+        const int col = gate * 8 + hh;
+        const float t = ((red[0][ml][col] + red[1][ml][col]) + (red[2][ml][col] + red[3][ml][col])) + a.bw[n0 + col];
+        pre[gate] = (a.sub_act == NBL_ACT_LINEAR ? t : nbl_act_apply(a.sub_act, t)) + a.gx[(size_t)m * a.Np + n0 + col];
+    }
+    const float gi = lstm_logistic(pre[0]);
+    const float gf = lstm_logistic(pre[1]);
+    const float gg = lstm_tanh(pre[2]);
+    const float go = lstm_logistic(pre[3]);
+    const size_t e = (size_t)m * a.H + h;
+    const float ig = __fmul_rn(gi, gg);
+    const float cf = __fmul_rn(a.c[e], gf);
+    const float ct = __fadd_rn(cf, ig);
+    a.c[e] = ct;
+    a.hout[e] = __fmul_rn(lstm_tanh(ct), go);
+}
+
 // LSTM cell for one time step from split-K partial sums of the recurrent GEMM:
 //   pre[gate] = sub_act(sum_z part[z][m][n] + bw[n]) + gx[m][n],  n = (h/32)*128 + gate*32 + h%32
 //   i, f, o = logistic(pre), g = tanh(pre);  c = c*f + i*g;  h_out = tanh(c)*o
@@ -229,23 +326,28 @@ __global__ void lstm_cell_kernel(const float *__restrict__ part, const float *__
     const int m = e / H, h = e - m * H;
     const int nbase = (h >> 5) * 128 + (h & 31);
     const size_t plane = (size_t)M * Np;
+    const float *__restrict__ p0 = part + (size_t)m * Np + nbase;
+    float acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+    #pragma unroll 8
+    for(int z = 0; z < S; z++) {
+        #pragma unroll
+        for(int gate = 0; gate < 4; gate++) acc[gate] += p0[(size_t)z * plane + gate * 32];
+    }
     float pre[4];
     #pragma unroll
     for(int gate = 0; gate < 4; gate++) {
-        const size_t at = (size_t)m * Np + nbase + gate * 32;
-        float acc = 0.0f;
-        for(int z = 0; z < S; z++) acc += part[(size_t)z * plane + at];
-        pre[gate] = nbl_act_apply(sub_act, acc + bw[nbase + gate * 32]) + gx[at];
+        const float t = acc[gate] + bw[nbase + gate * 32];
+        pre[gate] = (sub_act == NBL_ACT_LINEAR ? t : nbl_act_apply(sub_act, t)) + gx[(size_t)m * Np + nbase + gate * 32];
     }
-    const float gi = nbl_act_apply(NBL_ACT_LOGISTIC, pre[0]);
-    const float gf = nbl_act_apply(NBL_ACT_LOGISTIC, pre[1]);
-    const float gg = nbl_act_apply(NBL_ACT_TANH, pre[2]);
-    const float go = nbl_act_apply(NBL_ACT_LOGISTIC, pre[3]);
+    const float gi = lstm_logistic(pre[0]);
+    const float gf = lstm_logistic(pre[1]);
+    const float gg = lstm_tanh(pre[2]);
+    const float go = lstm_logistic(pre[3]);
     const float ig = __fmul_rn(gi, gg);
     const float cf = __fmul_rn(c[e], gf);
     const float ct = __fadd_rn(cf, ig);
     c[e] = ct;
-    h_out[e] = __fmul_rn(nbl_act_apply(NBL_ACT_TANH, ct), go);
+    h_out[e] = __fmul_rn(lstm_tanh(ct), go);
 }
 
 bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
@@ -266,6 +368,7 @@ struct nbl_lstm_plan {
     float *bu_dev, *bw_dev;             // [4*Hp] biases (BN shift folded in); for a linear sub_act bw is folded into bu
     float *gx_dev; float *h0_dev; float *c_dev; size_t gx_bytes, state_bytes;
     float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
+    unsigned G;                           // gate interleave: row of (gate, h) = (h/G)*4G + gate*G + h%G; 8 = single-launch steps
 };
 
 namespace {
@@ -396,6 +499,7 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
     nbl_lstm_plan *p = new nbl_lstm_plan();
     memset(p, 0, sizeof(*p));
     p->I = I; p->H = H; p->Hp = nbl_div_up(H, 32) * 32; p->sub_act = sub_act;
+    p->G = H % 128 == 0 ? 8 : 32;
     const unsigned Np = 4 * p->Hp;
     std::vector<float> ucat((size_t)Np * I, 0.0f), wcat((size_t)Np * H, 0.0f), bu(Np, 0.0f), bw(Np, 0.0f);
     std::vector<float> g(H), b(H);
@@ -408,7 +512,7 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
             nbl_fold_batchnorm(bias_host[s], scale_host ? scale_host[s] : NULL, mean_host ? mean_host[s] : NULL,
                                var_host ? var_host[s] : NULL, H, g.data(), b.data());
             for(unsigned h = 0; h < H; h++) {
-                const size_t row = (size_t)(h / 32) * 128 + gate * 32 + (h % 32);
+                const size_t row = (size_t)(h / p->G) * (4 * p->G) + gate * p->G + (h % p->G);
                 const float *src = weight_host[s] + (size_t)h * fan_in;
                 float *dst = cat.data() + row * fan_in;
                 // batchnorm scale folded into the row (1 when batch_normalize=0)
@@ -473,15 +577,31 @@ int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_de
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
     if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
                        p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
-    // Recurrent half.  One step is only [B x H].[H x 4H]: to put work on every CU the k range is split
-    // over blockIdx.z into partial sums (deterministic order) and a small cell kernel finishes the step.
-    // Narrow problems keep the single fused kernel.  h_{t-1} is read straight from y[t-1].
+    const size_t step = (size_t)B * p->H;
+    if(p->G == 8) {
+        // Recurrent half, one launch per step (lstm_step_kernel).  h_{t-1} is read straight from y[t-1].
+        if(!aligned16(y_dev) || !aligned16(p->wcat_dev) || !aligned16(p->h0_dev))
+            return nbl_fail(ctx, NBL_EINVAL, "nbl_lstm_fwd: y_dev must be 16-byte aligned");
+        LstmStepArgs sa;
+        sa.w = p->wcat_dev; sa.bw = p->bw_dev; sa.c = p->c_dev; sa.B = (int)B; sa.H = (int)p->H; sa.Np = (int)Np;
+        sa.sub_act = p->sub_act;
+        const dim3 grid(Np / 32, nbl_div_up(B, 32));
+        for(unsigned t = 0; t < T; t++) {
+            sa.hprev = t == 0 ? p->h0_dev : y_dev + (size_t)(t - 1) * step;
+            sa.gx = p->gx_dev + (size_t)t * B * Np;
+            sa.hout = y_dev + (size_t)t * step;
+            hipLaunchKernelGGL(lstm_step_kernel, grid, dim3(256), 0, ctx->stream, sa);
+            NBL_LAUNCH_CHECK(ctx, "lstm_step_kernel");
+        }
+    } else {
+    // Recurrent half for the 32-wide gate interleave.  One step is only [B x H].[H x 4H]: to put work on
+    // every CU the k range is split over blockIdx.z into partial sums (deterministic order) and a small
+    // cell kernel finishes the step.  Narrow problems keep the single fused kernel.
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.Bw = p->wcat_dev; a.M = (int)B; a.N = (int)Np; a.K = (int)p->H; a.lda = (int)p->H; a.ldb = (int)p->H;
     a.ldc = (int)Np;
     a.b = p->bw_dev; a.act = p->sub_act; a.c = p->c_dev; a.H = (int)p->H;
-    const size_t step = (size_t)B * p->H;
     const int ktiles = nbl_div_up(p->H, GEMM_BK);
     const unsigned gm = nbl_div_up(B, 64), gn = Np / 128;
     int S = 1;
@@ -515,6 +635,7 @@ int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_de
             hipLaunchKernelGGL((gemm_nt_kernel<1, 4, 2, 1, EPI_LSTM>), grid, dim3(128), 0, ctx->stream, a);
             NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(lstm)");
         }
+    }
     }
     if(cell_dev)
         NBL_HIP(ctx, hipMemcpyAsync(cell_dev, p->c_dev, st_need, hipMemcpyDeviceToDevice, ctx->stream));

@@ -210,20 +210,26 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-__global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
-    __shared__ float red[4];
+// One block of THREADS threads per row (long rows take 1024 threads: the exp is double precision and
+// there are only as many blocks as rows).
+template<int THREADS>
+__global__ __launch_bounds__(THREADS) void softmax_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
+    constexpr int WAVES = THREADS / 64;
+    __shared__ float red[WAVES];
     const float *in = x + (size_t)blockIdx.x * n;
     float *out = y + (size_t)blockIdx.x * n;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     float m = -FLT_MAX;
-    for(unsigned j = tid; j < n; j += 256) m = fmaxf(m, in[j]);
+    for(unsigned j = tid; j < n; j += THREADS) m = fmaxf(m, in[j]);
     m = wave_max(m);
     if(lane == 0) red[wave] = m;
     __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    m = red[0];
+    #pragma unroll
+    for(int w = 1; w < WAVES; w++) m = fmaxf(m, red[w]);
     __syncthreads();
     float s = 0.0f;
-    for(unsigned j = tid; j < n; j += 256) {
+    for(unsigned j = tid; j < n; j += THREADS) {
         const float e = (float)exp((double)(in[j] - m));
         out[j] = e;
         s += e;
@@ -231,8 +237,16 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ 
     s = wave_sum(s);
     if(lane == 0) red[wave] = s;
     __syncthreads();
-    s = (red[0] + red[1]) + (red[2] + red[3]);
-    for(unsigned j = tid; j < n; j += 256) out[j] = out[j] / s;
+    // pairwise over the waves, the same tree for every thread
+    float part[WAVES];
+    #pragma unroll
+    for(int w = 0; w < WAVES; w++) part[w] = red[w];
+    #pragma unroll
+    for(int width = WAVES / 2; width >= 1; width /= 2)
+        #pragma unroll
+        for(int w = 0; w < width; w++) part[w] = part[2 * w] + part[2 * w + 1];
+    s = part[0];
+    for(unsigned j = tid; j < n; j += THREADS) out[j] = out[j] / s;
 }
 
 // ---- elementwise ---------------------------------------------------------------------------------
@@ -377,7 +391,8 @@ int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned row
     if(!ctx) return NBL_EINVAL;
     NBL_REQUIRE(ctx, x_dev && y_dev, "nbl_softmax_fwd: NULL pointer");
     if(rows == 0 || n == 0) return NBL_OK;
-    hipLaunchKernelGGL(softmax_kernel, dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    if(n > 2048) hipLaunchKernelGGL(softmax_kernel<1024>, dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
+    else         hipLaunchKernelGGL(softmax_kernel<256>, dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
     NBL_LAUNCH_CHECK(ctx, "softmax_kernel");
     return NBL_OK;
 }

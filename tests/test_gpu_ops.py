@@ -319,7 +319,10 @@ def test_softmax(ctx, shape):
 
 
 LSTM = [(3, 2, 5, 4, False, "linear"), (4, 3, 6, 5, True, "tanh"), (6, 8, 64, 96, False, "linear"),
-        (5, 64, 128, 128, True, "linear"), (3, 70, 40, 33, False, "linear")]
+        (5, 64, 128, 128, True, "linear"), (3, 70, 40, 33, False, "linear"),
+        # hidden sizes that are multiples of 128 take the one-launch-per-step kernel: ragged batch tiles,
+        # a non-linear sub-layer activation, odd and even numbers of load batches per wave
+        (4, 37, 96, 256, False, "tanh"), (3, 33, 64, 384, True, "linear"), (2, 5, 48, 512, False, "linear")]
 
 
 @pytest.mark.parametrize("case", LSTM)
