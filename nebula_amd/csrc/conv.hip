@@ -1,21 +1,28 @@
 // Convolution forward as an implicit GEMM on the fp32 matrix cores of gfx950.
 //
-//   Y[f][n] = sum_kk  Wp[kk][f] * patch(kk, n)        f < F,  n = (b, oh, ow),  kk = (c, i, j)
+//   Y[f][n] = sum_kk  Wp[kk][f] * patch(kk, n)        f < F,  n = (b, oh, ow),  kk = a (c, i, j)
 //
 // The patch matrix (what im2col would write, common/utils.cc:81-119) is never stored: each block
-// gathers its BK x BN slice straight from the NCHW input into LDS.  The gather is driven by a small
-// per-layer table, one entry per kk, holding the input offset c*H*W + i*W + j and the tap (i, j);
-// a pixel column n contributes its base offset and its top-left input coordinate.  The same device
-// function feeds nbl_im2col, so the index map can be compared element for element with the CPU one.
+// gathers its BK x BN slice straight from the NCHW input into LDS.  The gather is driven by small
+// per-layer tables: one entry per patch row holding the input offset c*H*W + i*W + j and the tap
+// (i, j), or, for layers whose rows are packed tap-major, one entry per k-tile; a pixel column n
+// contributes its base offset and its top-left input coordinate.  The same device function feeds
+// nbl_im2col, so the index map can be compared element for element with the CPU one.
 //
 // Tiling: a block of 64*WAVES_M*WAVES_N threads owns a BM x BN tile of Y; each wave owns
 // (MT*32) x (NT*32) of it as MT*NT accumulators of v_mfma_f32_32x32x2_f32.  Filters are the MFMA
-// rows and pixels the MFMA columns, so that the 32 lanes holding one accumulator row write 32
+// rows and pixels the MFMA columns, so that the 32 lanes holding one accumulator row write 32*NT
 // consecutive pixels of one output plane.  Both operands sit in LDS k-major ([k][m] and [k][n]):
-// lanes 0-31 read 32 consecutive floats of row k, lanes 32-63 of row k+1 (one ds_read_b32 per
-// operand per MFMA, which the 64-cycle fp32 MFMA hides easily).  Weights are re-laid out once, at
-// pack time, to [Kp][Mp] so their tile loads are contiguous float4s.  LDS is double buffered with
-// register staging: the loads of tile t+1 are issued before the MFMAs of tile t.
+// lanes 0-31 read row k, lanes 32-63 row k+1, each lane its MT (NT) adjacent values in one read.
+// Weights are re-laid out once, at pack time, to [Kp][Mp] so their tile loads are contiguous
+// float4s.  LDS is double buffered and fed through two register stages: the global loads of
+// k-tile t+2 are issued before the MFMAs of k-tile t.
+//
+// Work distribution: one block per output tile, except that the tiles of an under-filled last round
+// may be cut into slices along k (one block per slice, raw sums to scratch, a finishing kernel adds
+// them in order and applies the epilogue); block indices are renumbered so that the filter tiles of
+// one pixel tile share an XCD.  The tile shape and whether to split are measured per (layer, batch)
+// on first use.
 #include "nbl_internal.h"
 
 #include <cmath>
@@ -257,8 +264,7 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.b[r] = buf_load(xres, off);
             }
         }
-        // the pipeline runs two k-tiles past the block's last one: those loads repeat the last weight tile
-        const float *__restrict__ wtile = a.wp + (size_t)min(kt, nkt - 1) * BK * a.Mp + ld_m0;
+        const float *__restrict__ wtile = a.wp + (size_t)kt * BK * a.Mp + ld_m0;
         {
             const int row = tid / (BM / 4), col4 = tid % (BM / 4);
             if(A_VEC >= NTHREADS || tid < A_VEC)
@@ -271,8 +277,8 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.a1 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
         }
     };
-    // issue the loads of the next k-tile; the table entries of the k-tile after it follow (the table ends
-    // in all-padding tiles for the pipeline's run past the last k-tile)
+    // issue the loads of the next k-tile; the table entries of the k-tile after it follow (the tables end
+    // in all-padding tiles, so the entry after the last k-tile exists)
     auto ld_next = [&](Stage &st) {
         load_tile(st, ld_kt);
         ++ld_kt;
@@ -704,7 +710,6 @@ struct nbl_conv_plan {
     bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 32)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
-    bool force_scalar_gather;   // tests: keep 1x1 layers on the table-driven gather
     int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so
     bool tuned_split;
     float *ws_dev; size_t ws_bytes;   // partial sums of split launches (grown on demand)
@@ -789,7 +794,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->K = C * ksize * ksize;
     p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
-    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1; p->force_scalar_gather = false;
+    p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
     p->split_mode = -1; p->tuned_split = false; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
@@ -904,9 +909,8 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
                          ((size_t)y_dev & 7) == 0 && (!rs || ((size_t)rs->res & 7) == 0)) ? 0 : sloped ? 2 : 1;
     a.ttab = p->ttab_dev; a.ksize = (int)p->k; a.plane_bytes = p->H * p->W * 4u;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
-    if(p->tap_major && !p->force_scalar_gather) gather = GATHER_TAP_MAJOR;
-    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 &&
-       !p->force_scalar_gather)
+    if(p->tap_major) gather = GATHER_TAP_MAJOR;
+    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0)
         gather = GATHER_1X1_VEC4;
     a.whole_tiles = (int)blocks; a.split = 1; a.n_start = 0; a.n_tail = 0; a.ws = NULL;
     size_t grid = blocks;

@@ -7,10 +7,10 @@
 //
 // LSTM (models/layers/lstm_layer.cc:233-346): the input half  U.x  is hoisted out of the time loop
 // (one GEMM over all T*B rows) and the recurrent half  W.h  runs once per step with the gate
-// non-linearities and the cell update in its epilogue.  The four gate matrices are interleaved at
-// pack time in blocks of 32 hidden units, so that the four 32x32 accumulators a wave owns are the
-// i, f, g, o pre-activations of the same (batch row, hidden unit) elements and the whole cell update
-// happens in registers.
+// non-linearities and the cell update fused behind it.  The four gate matrices are interleaved at
+// pack time (8 hidden units wide when H % 128 == 0: lstm_step_kernel, one launch per step; 32 wide
+// otherwise), so that the i, f, g, o pre-activations of one (batch row, hidden unit) sit in one MFMA
+// tile or in the four tiles of one wave.
 //
 // LDS layout: [row][BK + 4] floats per operand.  A k-tile of 32 is consumed by 16 MFMAs; lanes 0-31
 // feed k = 0..15 and lanes 32-63 feed k = 16..31 (any pairing of k values is legal as long as both
