@@ -147,12 +147,35 @@ def single_conv(args):
     ctx.close()
 
 
+def image_input(args):
+    """Device-side image preprocessing (nbl_image_to_input): 64 byte images of 375x500x3 -> 3x224x224 float planes."""
+    from nebula_amd import hip
+    ctx = hip.Ctx(0)
+    B = args.batch or 64
+    rng = np.random.default_rng(1)
+    imgs = ctx.array(rng.integers(0, 256, (B, 375, 500, 3), dtype=np.uint8), dtype=np.uint8)
+    for _ in range(args.warmup):
+        out = ctx.image_to_input(imgs, 224, 224)
+        out.free()
+    out = ctx.empty((B, 3, 224, 224))
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        ctx.check(hip.lib().nbl_image_to_input(ctx.h, imgs.ptr, B, 375, 500, 3, out.ptr, 224, 224))
+    ms = ctx.timer_stop() / args.steps
+    # every output pixel reads 4 source pixels of 3 bytes and writes 3 floats; compulsory traffic is the two tensors
+    print(json.dumps({"metric": "image preprocessing images/s", "value": round(B / ms * 1e3, 1), "unit": "images/s",
+                      "ms_per_launch": round(ms, 4), "bytes_in": int(imgs.nbytes), "bytes_out": int(out.nbytes),
+                      "GBps": round((imgs.nbytes + out.nbytes) / ms / 1e6, 1), "steps": args.steps}), flush=True)
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv", "images"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
                          "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
                          "for counter passes over a single kernel")
@@ -171,6 +194,8 @@ def main():
         return copy_calibration(args)
     if args.workload == "conv":
         return single_conv(args)
+    if args.workload == "images":
+        return image_input(args)
 
     from nebula_amd.net import Network
 

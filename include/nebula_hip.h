@@ -178,6 +178,16 @@ int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev,
                      unsigned in_c, unsigned in_h, unsigned in_w,
                      unsigned out_c, unsigned out_h, unsigned out_w, int act);
 
+/* ---- image input contract ---------------------------------------------------------------------------
+ * The preprocessing of convolutional_t::load_data (models/networks/convolutional.cc:384-412) on the
+ * device, so that a batch travels over PCIe as bytes: `images` 8-bit interleaved images
+ * [src_h][src_w][channels] (channel order as decoded, B G R) -> planes [images][channels][dst_h][dst_w]
+ * of byte / 255.0 with planes 0 and 2 swapped; when the sizes differ the image is first resized as
+ * cv::resize(..., cv::INTER_LINEAR) does for 8-bit data (OpenCV's fixed-point bilinear arithmetic,
+ * restated from its published algorithm: OpenCV itself is not available to check against). */
+int nbl_image_to_input(nbl_ctx *ctx, const unsigned char *src_dev, unsigned images, unsigned src_h, unsigned src_w,
+                       unsigned channels, float *dst_dev, unsigned dst_h, unsigned dst_w);
+
 /* softmax_layer_t::_forward_() (models/layers/softmax_layer.cu:30-41; CPU twin softmax_layer.cc:85-106). */
 int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned rows, unsigned n);
 

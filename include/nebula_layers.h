@@ -46,6 +46,11 @@ int nbl_net_layer_info(nbl_net *net, int layer, unsigned *info);
 int nbl_net_layer_flop(nbl_net *net, int layer, double *flop_per_row);
 /* host -> device input, [batch_size][input_size] floats */
 int nbl_net_set_input(nbl_net *net, const float *host, size_t count);
+/* The image driver's load_data() (models/networks/convolutional.cc:384-412) with the preprocessing on the
+ * device: `images` (= batch size) 8-bit interleaved images [height][width][channels] in decoded channel
+ * order (B, G, R) are copied as bytes, resized to the network's input size if they differ (8-bit
+ * INTER_LINEAR), scaled by 1/255 and stored as planes with planes 0 and 2 swapped. */
+int nbl_net_set_input_images(nbl_net *net, const unsigned char *host, unsigned images, unsigned height, unsigned width);
 /* network_t::forward(); asynchronous unless the net ends in a softmax (which copies to the host) */
 int nbl_net_forward(nbl_net *net);
 int nbl_net_sync(nbl_net *net);

@@ -85,6 +85,7 @@ int nbl_ctx_destroy(nbl_ctx *ctx) {
     hipStreamSynchronize(ctx->stream);
     if(ctx->ev_start) hipEventDestroy(ctx->ev_start);
     if(ctx->ev_stop) hipEventDestroy(ctx->ev_stop);
+    if(ctx->rz_tab_dev) hipFree(ctx->rz_tab_dev);
     if(ctx->owns_stream) hipStreamDestroy(ctx->stream);
     delete ctx;
     return NBL_OK;

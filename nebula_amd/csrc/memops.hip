@@ -2,6 +2,9 @@
 // inference batchnorm.  Each kernel reads its input once and writes its output once; wherever the
 // layout allows, a lane moves 16 bytes per access.
 #include "nbl_internal.h"
+#include <cmath>
+#include <vector>
+#include <algorithm>
 
 #include <cfloat>
 
@@ -284,6 +287,64 @@ __global__ void batchnorm_inference_kernel(float *__restrict__ y, const float *_
     y[e] = __fmul_rn(normed, scale[c]);
 }
 
+
+// ---- image input contract ---------------------------------------------------------------------------
+// 8-bit interleaved images -> network input planes: optional bilinear resize in OpenCV's 8-bit
+// fixed-point arithmetic (weights are shorts scaled by 2048, horizontal pass in int, vertical pass
+// ((b0 * (S0 >> 4)) >> 16) + ((b1 * (S1 >> 4)) >> 16) + 2) >> 2), then byte / 255.0 and planes 0 and 2
+// swapped (models/networks/convolutional.cc:384-412).  One thread per output pixel; the tap tables are
+// built on the host.  tab = [xofs | x weights (a0 | a1 << 16) | row0 | row1 | y weights] as ints.
+__global__ void image_to_input_kernel(const unsigned char *__restrict__ src, float *__restrict__ dst,
+                                      const int *__restrict__ tab, unsigned images, int src_h, int src_w, int ch,
+                                      int dst_h, int dst_w, int resize) {
+    const int dx = blockIdx.x * blockDim.x + threadIdx.x, dy = blockIdx.y, img = blockIdx.z;
+    if(dx >= dst_w) return;
+    const unsigned char *__restrict__ in = src + (size_t)img * src_h * src_w * ch;
+    float *__restrict__ out = dst + (size_t)img * ch * dst_h * dst_w;
+    const size_t plane = (size_t)dst_h * dst_w;
+    int sx = dx, sx1 = dx, a0 = 2048, a1 = 0, r0 = dy, r1 = dy, b0 = 2048, b1 = 0;
+    if(resize) {
+        sx = tab[dx];
+        sx1 = sx + 1 < src_w ? sx + 1 : sx;
+        const int aw = tab[dst_w + dx];
+        a0 = (short)(aw & 0xffff); a1 = (short)(aw >> 16);
+        r0 = tab[2 * dst_w + dy]; r1 = tab[2 * dst_w + dst_h + dy];
+        const int bw = tab[2 * dst_w + 2 * dst_h + dy];
+        b0 = (short)(bw & 0xffff); b1 = (short)(bw >> 16);
+    }
+    for(int c = 0; c < ch; c++) {
+        int v;
+        if(resize) {
+            const int S0 = in[((size_t)r0 * src_w + sx) * ch + c] * a0 + in[((size_t)r0 * src_w + sx1) * ch + c] * a1;
+            const int S1 = in[((size_t)r1 * src_w + sx) * ch + c] * a0 + in[((size_t)r1 * src_w + sx1) * ch + c] * a1;
+            v = (((b0 * (S0 >> 4)) >> 16) + ((b1 * (S1 >> 4)) >> 16) + 2) >> 2;
+            v = v < 0 ? 0 : v > 255 ? 255 : v;
+        } else {
+            v = in[((size_t)dy * src_w + dx) * ch + c];
+        }
+        const int cp = ch >= 3 && c == 0 ? 2 : ch >= 3 && c == 2 ? 0 : c;      // planes 0 and 2 change places
+        out[cp * plane + (size_t)dy * dst_w + dx] = (float)((double)v / 255.0);
+    }
+}
+
+// Source index and the two weights of every destination coordinate along one axis.
+static void linear_taps(unsigned dst_n, unsigned src_n, bool clamp_weight, std::vector<int> &ofs, std::vector<int> &weights) {
+    ofs.resize(dst_n); weights.resize(dst_n);
+    const double scale = (double)src_n / (double)dst_n;
+    for(unsigned d = 0; d < dst_n; d++) {
+        float f = (float)((d + 0.5) * scale - 0.5);
+        int s = (int)std::floor((double)f);
+        f -= (float)s;
+        if(clamp_weight) {
+            if(s < 0) { f = 0.0f; s = 0; }
+            if(s >= (int)src_n - 1) { f = 0.0f; s = (int)src_n - 1; }
+        }
+        const int w0 = (int)std::nearbyint((double)((1.0f - f) * 2048.0f)), w1 = (int)std::nearbyint((double)(f * 2048.0f));
+        ofs[d] = s;
+        weights[d] = (w0 & 0xffff) | (w1 << 16);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -431,6 +492,36 @@ int nbl_batchnorm_inference(nbl_ctx *ctx, float *y_dev, const float *mean_dev, c
     hipLaunchKernelGGL(batchnorm_inference_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
                        y_dev, mean_dev, var_dev, scale_dev, total, channel, size);
     NBL_LAUNCH_CHECK(ctx, "batchnorm_inference_kernel");
+    return NBL_OK;
+}
+
+int nbl_image_to_input(nbl_ctx *ctx, const unsigned char *src_dev, unsigned images, unsigned src_h, unsigned src_w,
+                       unsigned channels, float *dst_dev, unsigned dst_h, unsigned dst_w) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, src_dev && dst_dev, "nbl_image_to_input: NULL pointer");
+    NBL_REQUIRE(ctx, src_h && src_w && channels && dst_h && dst_w, "nbl_image_to_input: zero dimension");
+    if(images == 0) return NBL_OK;
+    if(images > 65535 || dst_h > 65535 || src_h >= (1u << 15) || src_w >= (1u << 15))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_image_to_input: more than 65535 images or rows, or a source side of 32768 or more");
+    const int resize = src_h != dst_h || src_w != dst_w;
+    if(resize && !(ctx->rz_tab_dev && ctx->rz_src_h == src_h && ctx->rz_src_w == src_w && ctx->rz_dst_h == dst_h && ctx->rz_dst_w == dst_w)) {
+        std::vector<int> xofs, xw, yofs, yw, tab;
+        linear_taps(dst_w, src_w, true, xofs, xw);
+        linear_taps(dst_h, src_h, false, yofs, yw);
+        tab.insert(tab.end(), xofs.begin(), xofs.end());
+        tab.insert(tab.end(), xw.begin(), xw.end());
+        for(unsigned k = 0; k < 2; k++)       // the two source rows of a destination row, clipped into the image
+            for(unsigned d = 0; d < dst_h; d++) tab.push_back(std::min(std::max(yofs[d] + (int)k, 0), (int)src_h - 1));
+        tab.insert(tab.end(), yw.begin(), yw.end());
+        int rc = nbl_free(ctx, ctx->rz_tab_dev);
+        ctx->rz_tab_dev = NULL;
+        if(rc != NBL_OK || (rc = nbl_malloc(ctx, (void**)&ctx->rz_tab_dev, tab.size() * sizeof(int))) != NBL_OK ||
+           (rc = nbl_h2d(ctx, ctx->rz_tab_dev, tab.data(), tab.size() * sizeof(int))) != NBL_OK) return rc;
+        ctx->rz_src_h = src_h; ctx->rz_src_w = src_w; ctx->rz_dst_h = dst_h; ctx->rz_dst_w = dst_w;
+    }
+    hipLaunchKernelGGL(image_to_input_kernel, dim3(nbl_div_up(dst_w, 256), dst_h, images), dim3(256), 0, ctx->stream,
+                       src_dev, dst_dev, ctx->rz_tab_dev, images, (int)src_h, (int)src_w, (int)channels, (int)dst_h, (int)dst_w, resize);
+    NBL_LAUNCH_CHECK(ctx, "image_to_input_kernel");
     return NBL_OK;
 }
 

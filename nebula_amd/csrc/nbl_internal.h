@@ -17,6 +17,9 @@ struct nbl_ctx {
     hipEvent_t ev_start, ev_stop;
     int num_cu;
     char err[512];
+    // tap tables of the last image resize geometry (nbl_image_to_input), kept on the device
+    unsigned rz_src_h, rz_src_w, rz_dst_h, rz_dst_w;
+    int *rz_tab_dev;
 };
 
 // Records a formatted message on the context and returns `code`.

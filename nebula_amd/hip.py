@@ -37,6 +37,7 @@ SIGNATURES = {
     "nbl_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
     "nbl_copy_d2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_sync": (C.c_int, [_vp]),
+    "nbl_image_to_input": (C.c_int, [_vp, _vp, _u, _u, _u, _u, _vp, _u, _u]),
     "nbl_conv2d_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, _u, _u, _u, _u, _u, C.c_int,
                                   C.POINTER(_vp)]),
     "nbl_conv2d_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
@@ -184,6 +185,13 @@ class Ctx:
 
     def sync(self):
         self.check(lib().nbl_sync(self.h))
+
+    def image_to_input(self, images_u8, dst_h, dst_w):
+        """images_u8: DeviceArray [n][h][w][c] of uint8 -> DeviceArray [n][c][dst_h][dst_w] of float32."""
+        n, h, w, c = images_u8.shape
+        out = self.empty((n, c, dst_h, dst_w))
+        self.check(lib().nbl_image_to_input(self.h, images_u8.ptr, n, h, w, c, out.ptr, dst_h, dst_w))
+        return out
 
     def copy(self, dst, src, nbytes=None):
         """Device-to-device copy kernel between two DeviceArrays."""

@@ -118,6 +118,10 @@ int nbl_net_set_input(nbl_net *n, const float *host, size_t count) {
     NBL_NET_TRY(if(!n || !host) throw std::runtime_error("NULL argument"); n->net->set_input(host, count));
 }
 
+int nbl_net_set_input_images(nbl_net *n, const unsigned char *host, unsigned images, unsigned height, unsigned width) {
+    NBL_NET_TRY(if(!n || !host) throw std::runtime_error("NULL argument"); n->net->set_input_images(host, images, height, width));
+}
+
 int nbl_net_forward(nbl_net *n) {
     NBL_NET_TRY(if(!n) throw std::runtime_error("NULL argument"); n->net->forward());
 }

@@ -64,7 +64,8 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false) {
+    last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false),
+    image_staging_dev(NULL), image_staging_bytes(0) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
@@ -79,6 +80,7 @@ inference_net_t::~inference_net_t() {
     for(size_t i = layers.size(); i > 0; i--) delete layers[i - 1];
     for(size_t i = 0; i < events.size(); i++) (void)hipEventDestroy((hipEvent_t)events[i]);
     if(input_data_dev && ctx) nbl_free(ctx, input_data_dev);
+    if(image_staging_dev && ctx) nbl_free(ctx, image_staging_dev);
     delete [] input_data;
     if(ctx) nbl_ctx_destroy(ctx);
 }
@@ -170,6 +172,24 @@ void inference_net_t::set_input(const float *host, size_t count) {
     if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     if(count != (size_t)batch_size * input_size) throw std::runtime_error("Error: input tensor has the wrong size");
     nbl_check(ctx, nbl_h2d(ctx, input_data_dev, host, count * sizeof(float)), "nbl_h2d(input)");
+}
+
+// The image driver's load_data() contract (models/networks/convolutional.cc:384-412) with the resize,
+// scaling and plane reordering done on the device: the batch crosses PCIe as bytes.
+void inference_net_t::set_input_images(const unsigned char *host, unsigned images, unsigned height, unsigned width) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
+    if(is_recurrent) throw std::runtime_error("Error: image input on a recurrent network");
+    if(images != batch_size) throw std::runtime_error("Error: input batch has the wrong number of images");
+    const size_t bytes = (size_t)images * height * width * input_channel;
+    if(bytes > image_staging_bytes) {
+        nbl_check(ctx, nbl_free(ctx, image_staging_dev), "nbl_free(image staging)");
+        image_staging_dev = NULL; image_staging_bytes = 0;
+        nbl_check(ctx, nbl_malloc(ctx, (void**)&image_staging_dev, bytes), "nbl_malloc(image staging)");
+        image_staging_bytes = bytes;
+    }
+    nbl_check(ctx, nbl_h2d(ctx, image_staging_dev, host, bytes), "nbl_h2d(images)");
+    nbl_check(ctx, nbl_image_to_input(ctx, image_staging_dev, images, height, width, input_channel, input_data_dev,
+                                      input_height, input_width), "nbl_image_to_input");
 }
 
 void inference_net_t::load_data(const unsigned) {}

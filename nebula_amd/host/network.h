@@ -78,6 +78,9 @@ public:
     void init_from_stream(std::istream &cfg, const std::string m_input_weight = "");
     // Copy a host tensor [batch_size][input_size] to the device input.
     void set_input(const float *host, size_t count);
+    // `images` 8-bit interleaved images [height][width][input_channel] (channel order B, G, R as decoded) ->
+    // network input, as convolutional_t::load_data() prepares it (resize, / 255, planes 0 and 2 swapped).
+    void set_input_images(const unsigned char *host, unsigned images, unsigned height, unsigned width);
     void run(const std::string m_output_weight = "");
     bool recurrent() const { return is_recurrent; }
 
@@ -106,6 +109,8 @@ private:
     int first_after_lstm;      // index of the first layer after the last LSTM, -1 if none
     unsigned batch_override;
     bool is_recurrent;
+    unsigned char *image_staging_dev;   // device copy of the last byte-image batch
+    size_t image_staging_bytes;
     std::vector<void*> events;
 };
 

@@ -26,6 +26,7 @@ SIGNATURES = {
     "nbl_net_layer_info": (C.c_int, [_vp, C.c_int, C.POINTER(_u)]),
     "nbl_net_layer_flop": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),
     "nbl_net_set_input": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "nbl_net_set_input_images": (C.c_int, [_vp, _vp, _u, _u, _u]),
     "nbl_net_forward": (C.c_int, [_vp]),
     "nbl_net_sync": (C.c_int, [_vp]),
     "nbl_net_forward_timed": (C.c_int, [_vp, C.POINTER(C.c_float)]),
@@ -126,6 +127,12 @@ class Network:
     def set_input(self, x):
         x = np.ascontiguousarray(x, np.float32)
         self._check(lib().nbl_net_set_input(self.h, x.ctypes.data, x.size))
+
+    def set_input_images(self, images_u8):
+        """uint8 [batch][height][width][channels], decoded channel order (B, G, R)."""
+        a = np.ascontiguousarray(images_u8, np.uint8)
+        n, h, w, _ = a.shape
+        self._check(lib().nbl_net_set_input_images(self.h, a.ctypes.data, n, h, w))
 
     def forward(self):
         self._check(lib().nbl_net_forward(self.h))

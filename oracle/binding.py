@@ -89,6 +89,8 @@ def oracle():
         lib.orc_avgpool_forward.argtypes = [_f32p, _f32p] + [_u] * 7
         lib.orc_shortcut_forward.argtypes = [_f32p, _f32p, _f32p] + [_u] * 8
         lib.orc_softmax_forward.argtypes = [_f32p, _f32p, _u, _u]
+        lib.orc_image_to_input.argtypes = [C.c_void_p, _u, _u, _u, _f32p, _u, _u]
+        lib.orc_resize_linear_u8.argtypes = [C.c_void_p, _u, _u, _u, C.c_void_p, _u, _u]
         pp = C.POINTER(_f32p)
         lib.orc_lstm_forward.argtypes = [_f32p, pp, pp, pp, pp, pp, _f32p, _f32p, _u, _u, _u, _u, _u]
         _oracle = lib
@@ -214,6 +216,23 @@ def shortcut_forward(prev, conn, act="linear"):
     _, ic, ih, iw = conn.shape
     out = np.empty_like(prev)
     oracle().orc_shortcut_forward(_fp(prev), _fp(conn), _fp(out), B, ic, ih, iw, oc, oh, ow, ACT[act])
+    return out
+
+
+def image_to_input(img, dst_h, dst_w):
+    """img: uint8 [h][w][c] -> float32 [c][dst_h][dst_w] (convolutional_t::load_data contract)."""
+    img = np.ascontiguousarray(img, np.uint8)
+    h, w, c = img.shape
+    out = np.empty((c, dst_h, dst_w), np.float32)
+    oracle().orc_image_to_input(img.ctypes.data, h, w, c, _fp(out), dst_h, dst_w)
+    return out
+
+
+def resize_linear_u8(img, dst_h, dst_w):
+    img = np.ascontiguousarray(img, np.uint8)
+    h, w, c = img.shape
+    out = np.empty((dst_h, dst_w, c), np.uint8)
+    oracle().orc_resize_linear_u8(img.ctypes.data, h, w, c, out.ctypes.data, dst_h, dst_w)
     return out
 
 

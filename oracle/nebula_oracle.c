@@ -380,6 +380,87 @@ void orc_softmax_forward(const float *x, float *y, unsigned rows, unsigned n) {
 }
 
 /* ---------------------------------------------------------------------------------------
+ * Input contract of the image driver, convolutional_t::load_data
+ * (models/networks/convolutional.cc:384-412): an 8-bit interleaved image (rows of
+ * width*channels bytes, channel order as decoded: B, G, R) is resized with
+ * cv::resize(..., cv::INTER_LINEAR) when its size differs from the network's, turned into
+ * planes  data[c][h][w] = byte / 255.0  (double division, rounded to float), and planes 0 and
+ * 2 are swapped.
+ *
+ * PARITY UNPINNED for the resize: cv::resize lives in OpenCV, which is neither vendored in
+ * the reference nor installed here, and the reference holds no image fixtures.  What
+ * follows restates the published 8-bit INTER_LINEAR algorithm of OpenCV's imgproc module
+ * (resize.cpp: pixel-centre mapping fx = (dx + 0.5) * scale - 0.5; horizontal and vertical
+ * weights as shorts scaled by 2048 with round-half-even; horizontal pass in int; vertical
+ * pass ((b0 * (S0 >> 4)) >> 16) + ((b1 * (S1 >> 4)) >> 16) + 2) >> 2).  Pinned only by
+ * mathematics: identity at equal size, constants stay constant, within one grey level of
+ * exact bilinear interpolation (tests/test_oracle_math.py).  The byte -> float planes and
+ * the plane swap are pinned bit for bit by their closed form.
+ * ------------------------------------------------------------------------------------- */
+static int orc_round_half_even(double v) { return (int)nearbyint(v); }   /* default rounding mode */
+
+static void orc_linear_taps(unsigned dst_n, unsigned src_n, int clamp_weight, int *ofs, short *w) {
+    const double scale = (double)src_n / (double)dst_n;
+    for(unsigned d = 0; d < dst_n; d++) {
+        float f = (float)((d + 0.5) * scale - 0.5);
+        int s = (int)floor((double)f);
+        f -= (float)s;
+        if(clamp_weight) {          /* horizontal taps: weight forced to 0 at the borders */
+            if(s < 0) { f = 0.0f; s = 0; }
+            if(s >= (int)src_n - 1) { f = 0.0f; s = (int)src_n - 1; }
+        }
+        ofs[d] = s;
+        w[2 * d] = (short)orc_round_half_even((double)((1.0f - f) * 2048.0f));
+        w[2 * d + 1] = (short)orc_round_half_even((double)(f * 2048.0f));
+    }
+}
+
+void orc_resize_linear_u8(const unsigned char *src, unsigned src_h, unsigned src_w, unsigned ch,
+                          unsigned char *dst, unsigned dst_h, unsigned dst_w) {
+    int *xofs = (int*)malloc(sizeof(int) * dst_w), *yofs = (int*)malloc(sizeof(int) * dst_h);
+    short *alpha = (short*)malloc(sizeof(short) * 2 * dst_w), *beta = (short*)malloc(sizeof(short) * 2 * dst_h);
+    orc_linear_taps(dst_w, src_w, 1, xofs, alpha);
+    orc_linear_taps(dst_h, src_h, 0, yofs, beta);
+    for(unsigned dy = 0; dy < dst_h; dy++) {
+        /* vertical taps: the two source rows are clipped into the image, the weights are not touched */
+        int r0 = yofs[dy], r1 = yofs[dy] + 1;
+        if(r0 < 0) r0 = 0; if(r0 > (int)src_h - 1) r0 = (int)src_h - 1;
+        if(r1 < 0) r1 = 0; if(r1 > (int)src_h - 1) r1 = (int)src_h - 1;
+        const int b0 = beta[2 * dy], b1 = beta[2 * dy + 1];
+        for(unsigned dx = 0; dx < dst_w; dx++) {
+            const int sx = xofs[dx], sx1 = sx + 1 < (int)src_w ? sx + 1 : sx;   /* weight is 0 where sx + 1 is outside */
+            const int a0 = alpha[2 * dx], a1 = alpha[2 * dx + 1];
+            for(unsigned c = 0; c < ch; c++) {
+                const int S0 = src[((size_t)r0 * src_w + sx) * ch + c] * a0 + src[((size_t)r0 * src_w + sx1) * ch + c] * a1;
+                const int S1 = src[((size_t)r1 * src_w + sx) * ch + c] * a0 + src[((size_t)r1 * src_w + sx1) * ch + c] * a1;
+                const int v = (((b0 * (S0 >> 4)) >> 16) + ((b1 * (S1 >> 4)) >> 16) + 2) >> 2;
+                dst[((size_t)dy * dst_w + dx) * ch + c] = (unsigned char)(v < 0 ? 0 : v > 255 ? 255 : v);
+            }
+        }
+    }
+    free(xofs); free(yofs); free(alpha); free(beta);
+}
+
+void orc_image_to_input(const unsigned char *src, unsigned src_h, unsigned src_w, unsigned ch,
+                        float *dst, unsigned dst_h, unsigned dst_w) {
+    const unsigned char *img = src;
+    unsigned char *tmp = NULL;
+    if(src_h != dst_h || src_w != dst_w) {
+        tmp = (unsigned char*)malloc((size_t)dst_h * dst_w * ch);
+        orc_resize_linear_u8(src, src_h, src_w, ch, tmp, dst_h, dst_w);
+        img = tmp;
+    }
+    const size_t plane = (size_t)dst_h * dst_w;
+    for(unsigned h = 0; h < dst_h; h++)
+        for(unsigned c = 0; c < ch; c++)
+            for(unsigned w = 0; w < dst_w; w++)
+                dst[c * plane + (size_t)h * dst_w + w] = (float)(img[((size_t)h * dst_w + w) * ch + c] / 255.0);
+    if(ch >= 3)     /* convolutional.cc:403-405 swaps plane 0 and plane 2 */
+        for(size_t i = 0; i < plane; i++) { const float t = dst[i]; dst[i] = dst[i + 2 * plane]; dst[i + 2 * plane] = t; }
+    free(tmp);
+}
+
+/* ---------------------------------------------------------------------------------------
  * LSTM, lstm_layer.cc:233-346.  Sub-layer slots in file order (lstm_layer.cc:194-206):
  *   0 iW  1 fW  2 oW  3 cW  4 iU  5 fU  6 oU  7 cU
  * Per step: every sub-layer runs a full connected forward (GEMM nt, [BN], bias, the section's

@@ -15,6 +15,10 @@
  *     README.md:34).  Its summation order is not pinned by anything in the reference, so
  *     GEMM-backed results are pinned through the reference's own CUSTOM_BLAS twin
  *     (common/gemm.h) exactly and through OpenBLAS only to 1e-5 relative.
+ *   - PARITY UNPINNED: orc_resize_linear_u8 (the cv::resize step of the image driver's input
+ *     contract).  OpenCV is not part of the reference tree and not installed; the function
+ *     restates OpenCV's published 8-bit INTER_LINEAR arithmetic and is held only to
+ *     mathematical checks (identity, constants, one grey level from exact bilinear).
  */
 #ifndef NEBULA_ORACLE_H
 #define NEBULA_ORACLE_H
@@ -88,6 +92,14 @@ void orc_shortcut_forward(const float *prev, const float *conn, float *out, unsi
                           unsigned out_c, unsigned out_h, unsigned out_w, unsigned act);
 /* models/layers/softmax_layer.cc:85-106 */
 void orc_softmax_forward(const float *x, float *y, unsigned rows, unsigned n);
+
+/* convolutional_t::load_data (models/networks/convolutional.cc:384-412): 8-bit interleaved image ->
+ * network input planes (resize if needed, / 255.0, planes 0 and 2 swapped).  The resize restates
+ * OpenCV's 8-bit INTER_LINEAR and is PARITY UNPINNED (OpenCV is absent; see the .c file). */
+void orc_resize_linear_u8(const unsigned char *src, unsigned src_h, unsigned src_w, unsigned ch,
+                          unsigned char *dst, unsigned dst_h, unsigned dst_w);
+void orc_image_to_input(const unsigned char *src, unsigned src_h, unsigned src_w, unsigned ch,
+                        float *dst, unsigned dst_h, unsigned dst_w);
 
 /* models/layers/lstm_layer.cc:233-346, first forward() on a fresh layer (zero h and c).
  * x is time-major [T][B][I]; y is [T][B][H].  The eight sub-layers come in *file* order

@@ -249,3 +249,25 @@ def test_fused_shortcut_on_golden_resnet(golden_dir):
             if info["kind"] == "convolutional_layer" and nxt == "shortcut_layer":
                 continue
             assert rel(net.output(i), g["out_%02d" % i]) <= TOL, (i, info["kind"])
+
+
+def test_network_input_from_byte_images():
+    """set_input_images == set_input of the CPU-preprocessed batch (the image driver's load_data contract)."""
+    from nebula_amd.net import Network
+    print("CASE byte-image input", flush=True)
+    rng = np.random.default_rng(23)
+    onet = ob.OracleNet(MINI_RESNET)
+    blob = _random_weights(onet.specs, rng)
+    imgs = rng.integers(0, 256, (4, 45, 52, 3), dtype=np.uint8)
+    x = np.stack([ob.image_to_input(im, 32, 32) for im in imgs])
+    with Network(MINI_RESNET) as net:
+        net.load_weight_blob(blob)
+        net.set_input(x)
+        net.forward()
+        a = [net.output(i) for i in range(net.num_layers)]
+        net.set_input(np.zeros_like(x))
+        net.set_input_images(imgs)
+        net.forward()
+        b = [net.output(i) for i in range(net.num_layers)]
+    for u, v in zip(a, b):
+        np.testing.assert_array_equal(u.view(np.uint32), v.view(np.uint32))

@@ -176,6 +176,27 @@ def test_activation_kernels(ctx, name):
         np.testing.assert_array_equal(got > 0, x > 0)               # the mask itself
 
 
+IMAGES = [(2, 13, 17, 3, 13, 17), (3, 40, 30, 3, 16, 12), (2, 31, 29, 3, 47, 18), (1, 8, 8, 3, 227, 227), (2, 64, 48, 1, 5, 5),
+          (1, 375, 500, 3, 224, 224)]
+
+
+@pytest.mark.parametrize("case", IMAGES)
+def test_image_to_input_bit_exact(ctx, case):
+    """Device-side image preprocessing (resize, / 255, plane swap) equals the CPU restatement bit for bit."""
+    announce("image_to_input", case)
+    n, h, w, c, dh, dw = case
+    rng = np.random.default_rng(sum(case))
+    imgs = rng.integers(0, 256, (n, h, w, c), dtype=np.uint8)
+    got = ctx.image_to_input(ctx.array(imgs, dtype=np.uint8), dh, dw).numpy()
+    for i in range(n):
+        want = ob.image_to_input(imgs[i], dh, dw)
+        np.testing.assert_array_equal(bits(got[i]), bits(want))
+    # same geometry again (cached tap tables), other pixels
+    imgs2 = rng.integers(0, 256, (n, h, w, c), dtype=np.uint8)
+    got2 = ctx.image_to_input(ctx.array(imgs2, dtype=np.uint8), dh, dw).numpy()
+    np.testing.assert_array_equal(bits(got2[0]), bits(ob.image_to_input(imgs2[0], dh, dw)))
+
+
 def test_copy_d2d(ctx):
     from nebula_amd import hip
     announce("copy_d2d")

@@ -200,3 +200,27 @@ def test_openblas_backend_matches_custom_gemm():
     finally:
         ob.use_custom_gemm()
         ob.set_threads(1)
+
+
+def test_image_input_contract_closed_form_and_resize_bounds():
+    """Byte -> plane conversion is a closed form; the resize restatement (parity unpinned: OpenCV is absent) must
+    at least be the identity at equal size, keep constants, and stay within one grey level of exact bilinear
+    interpolation with pixel-centre alignment (torch, align_corners=False, no antialias)."""
+    rng = np.random.default_rng(3)
+    img = rng.integers(0, 256, (13, 17, 3), dtype=np.uint8)
+    got = ob.image_to_input(img, 13, 17)
+    want = (img.astype(np.float64) / 255.0).astype(np.float32).transpose(2, 0, 1)[[2, 1, 0]]
+    np.testing.assert_array_equal(got.view(np.uint32), np.ascontiguousarray(want).view(np.uint32))
+    np.testing.assert_array_equal(ob.resize_linear_u8(img, 13, 17), img)
+    const = np.full((9, 11, 3), 137, np.uint8)
+    np.testing.assert_array_equal(ob.resize_linear_u8(const, 20, 7), np.full((20, 7, 3), 137, np.uint8))
+    for (h, w, dh, dw) in [(13, 17, 26, 34), (40, 30, 16, 12), (31, 29, 47, 18), (8, 8, 227, 227), (64, 48, 5, 5)]:
+        src = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+        got = ob.resize_linear_u8(src, dh, dw).astype(np.float64)
+        t = torch.from_numpy(src.astype(np.float64)).permute(2, 0, 1)[None]
+        exact = torch.nn.functional.interpolate(t, size=(dh, dw), mode="bilinear", align_corners=False, antialias=False)
+        exact = exact[0].permute(1, 2, 0).numpy()
+        assert np.abs(got - exact).max() <= 1.0 + 1e-9, (h, w, dh, dw, np.abs(got - exact).max())
+        assert np.abs(got - exact).mean() < 0.35
+    gray = rng.integers(0, 256, (10, 12, 1), dtype=np.uint8)
+    np.testing.assert_array_equal(ob.image_to_input(gray, 10, 12)[0], (gray[..., 0] / 255.0).astype(np.float32))
