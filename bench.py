@@ -170,12 +170,55 @@ def image_input(args):
     ctx.close()
 
 
+def recurrent_driver(args):
+    """The recurrent driver's test step (models/networks/recurrent.cc): one-hot words of a 10000-word vocabulary,
+    T = 64 steps x `batch` sequences, 2 x LSTM 1024, projection + softmax on every row, perplexity update.
+    Timed twice: one-hot rows as token indices (gather), and as the dense [T*B x 10000] matrix the reference builds."""
+    from nebula_amd import zoo
+    from nebula_amd.net import Network
+    B = args.batch or 64
+    T, V, H = 64, 10000, 1024
+    rng = np.random.default_rng(5)
+    cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=2, classes=V)
+    net = Network(cfg)
+    net.load_weight_blob(make_weights(net.weight_layout(), rng, "lstm"))
+    net.softmax_copy(False)              # the probabilities stay on the device; the perplexity sum is computed there
+    tokens = rng.integers(0, V, (T, B)).astype(np.uint32)
+    labels = np.roll(tokens.ravel(), -1).reshape(T, B)
+    out = {}
+    for mode in ("tokens", "dense one-hot"):
+        if mode == "tokens":
+            net.set_input_tokens(tokens)
+        else:
+            x = np.zeros((T * B, V), np.float32)
+            x[np.arange(T * B), tokens.ravel()] = 1.0
+            net.set_input(x)
+        for _ in range(args.warmup):
+            net.forward()
+            ppl = net.accumulate_perplexity(labels)
+        net.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            net.forward()
+            ppl = net.accumulate_perplexity(labels)
+        net.sync()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        layer_ms = np.array(net.forward_timed())
+        out[mode] = {"ms_per_step": round(ms, 3), "sequences_per_s": round(B / ms * 1e3, 1), "words_per_s": round(T * B / ms * 1e3),
+                     "layer_ms": [round(float(v), 3) for v in layer_ms], "perplexity_figure": round(float(ppl), 2)}
+        log(mode, out[mode])
+    net.close()
+    print(json.dumps({"metric": "recurrent driver step (PTB shape) sequences/s", "value": out["tokens"]["sequences_per_s"],
+                      "unit": "sequences/s", "batch": B, "time_steps": T, "vocabulary": V, "steps": args.steps,
+                      "tokens": out["tokens"], "dense_one_hot": out["dense one-hot"]}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv", "images"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv", "images", "ptb"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
                          "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
                          "for counter passes over a single kernel")
@@ -196,6 +239,8 @@ def main():
         return single_conv(args)
     if args.workload == "images":
         return image_input(args)
+    if args.workload == "ptb":
+        return recurrent_driver(args)
 
     from nebula_amd.net import Network
 

@@ -156,6 +156,18 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
                   unsigned I, unsigned H, int sub_act, nbl_lstm_plan **out);
 int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *plan, const float *x_dev, float *y_dev, float *cell_dev,
                  unsigned T, unsigned B);
+/* The same layer fed by the recurrent driver's one-hot rows (models/networks/recurrent.cc:179-204, one 1.0
+ * per row of input_size = vocabulary entries), given as the position of that 1: tokens_dev[T*B], time-major.
+ * The input-side product  x . U^T  is then a gather of T*B columns of U (rows of a transposed copy the plan
+ * builds on first use) instead of a [T*B x V].[V x 4H] GEMM; same values as nbl_lstm_fwd on the one-hot
+ * matrix.  A token >= input_size stands for an all-zero row. */
+int nbl_lstm_fwd_tokens(nbl_ctx *ctx, nbl_lstm_plan *plan, const unsigned *tokens_dev, float *y_dev, float *cell_dev,
+                        unsigned T, unsigned B);
+/* sum_dev[0] = sum over rows of probs[row][targets[row]]: the quantity recurrent_t::print_results()
+ * accumulates into cumulative_cost with one-hot labels (models/networks/recurrent.cc:239-241); the driver's
+ * "perplexity" is exp(-log2(cumulative_cost / rows_seen)) (:247).  Deterministic summation order. */
+int nbl_target_prob_sum(nbl_ctx *ctx, const float *probs_dev, const unsigned *targets_dev, unsigned rows, unsigned n,
+                        float *sum_dev);
 int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *plan);
 
 /* ---- memory-bound layers -----------------------------------------------------------------------

@@ -51,6 +51,14 @@ int nbl_net_set_input(nbl_net *net, const float *host, size_t count);
  * order (B, G, R) are copied as bytes, resized to the network's input size if they differ (8-bit
  * INTER_LINEAR), scaled by 1/255 and stored as planes with planes 0 and 2 swapped. */
 int nbl_net_set_input_images(nbl_net *net, const unsigned char *host, unsigned images, unsigned height, unsigned width);
+/* recurrent_t::load_data() (models/networks/recurrent.cc:179-204) without the one-hot matrix: tokens[T*B]
+ * (time-major; = batch_size entries) name the position of the 1.0 in each input row.  Needs an [lstm] as the
+ * first layer, which then gathers weight columns instead of multiplying.  nbl_net_set_input switches back. */
+int nbl_net_set_input_tokens(nbl_net *net, const unsigned *host, size_t count);
+/* recurrent_t::print_results(), test branch (recurrent.cc:239-247): after a forward, adds the output layer's
+ * probabilities of the label tokens (one per output row) to the running sum and returns the driver's figure
+ * exp(-log2(sum / rows seen)). */
+int nbl_net_accumulate_perplexity(nbl_net *net, const unsigned *label_tokens, size_t count, float *perplexity);
 /* network_t::forward(); asynchronous unless the net ends in a softmax (which copies to the host) */
 int nbl_net_forward(nbl_net *net);
 int nbl_net_sync(nbl_net *net);

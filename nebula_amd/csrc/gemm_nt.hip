@@ -350,6 +350,38 @@ __global__ void lstm_cell_kernel(const float *__restrict__ part, const float *__
     h_out[e] = __fmul_rn(lstm_tanh(ct), go);
 }
 
+// dst[c][r] = src[r][c] through a 32x33 LDS tile (both sides coalesced).
+__global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, unsigned rows, unsigned cols) {
+    __shared__ float tile[32][33];
+    const unsigned c0 = blockIdx.x * 32, r0 = blockIdx.y * 32, tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for(unsigned j = ty; j < 32; j += 8)
+        if(r0 + j < rows && c0 + tx < cols) tile[j][tx] = src[(size_t)(r0 + j) * cols + c0 + tx];
+    __syncthreads();
+    for(unsigned j = ty; j < 32; j += 8)
+        if(c0 + j < cols && r0 + tx < rows) dst[(size_t)(c0 + j) * rows + r0 + tx] = tile[tx][j];
+}
+
+// Input half of an LSTM whose input rows are one-hot (the recurrent driver's encoding,
+// models/networks/recurrent.cc:179-204): x . Ucat^T is then column token[row] of Ucat, i.e. row
+// token[row] of its transpose, so the [T*B x V].[V x 4H] product becomes a gather of T*B rows:
+//   gx[row][n] = sub_act(UcatT[token[row]][n] + bu[n])
+// (the same single float add the GEMM epilogue performs on a sum whose other terms are zero).
+__global__ void lstm_token_gather_kernel(const float *__restrict__ ucat_t, const unsigned *__restrict__ tokens,
+                                         const float *__restrict__ bu, float *__restrict__ gx,
+                                         unsigned Np, unsigned vocab, int sub_act) {
+    const unsigned row = blockIdx.x, tok = tokens[row];
+    const float4 *__restrict__ src = reinterpret_cast<const float4*>(ucat_t + (size_t)tok * Np);
+    const float4 *__restrict__ b4 = reinterpret_cast<const float4*>(bu);
+    float4 *__restrict__ out = reinterpret_cast<float4*>(gx + (size_t)row * Np);
+    for(unsigned i = threadIdx.x; i < Np / 4; i += blockDim.x) {
+        float4 v = tok < vocab ? src[i] : make_float4(0.f, 0.f, 0.f, 0.f);     // a token outside the vocabulary is an all-zero row
+        const float4 b = b4[i];
+        v.x = nbl_act_apply(sub_act, v.x + b.x); v.y = nbl_act_apply(sub_act, v.y + b.y);
+        v.z = nbl_act_apply(sub_act, v.z + b.z); v.w = nbl_act_apply(sub_act, v.w + b.w);
+        out[i] = v;
+    }
+}
+
 bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
 
 }  // namespace
@@ -368,6 +400,7 @@ struct nbl_lstm_plan {
     float *bu_dev, *bw_dev;             // [4*Hp] biases (BN shift folded in); for a linear sub_act bw is folded into bu
     float *gx_dev; float *h0_dev; float *c_dev; size_t gx_bytes, state_bytes;
     float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
+    float *ucat_t_dev;                    // [I][4*Hp] transpose of ucat_dev, built on the first token-input forward
     unsigned G;                           // gate interleave: row of (gate, h) = (h/G)*4G + gate*G + h%G; 8 = single-launch steps
 };
 
@@ -544,17 +577,17 @@ int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->ucat_dev); nbl_free(ctx, p->wcat_dev); nbl_free(ctx, p->bu_dev); nbl_free(ctx, p->bw_dev);
     nbl_free(ctx, p->gx_dev); nbl_free(ctx, p->h0_dev); nbl_free(ctx, p->c_dev); nbl_free(ctx, p->part_dev);
+    nbl_free(ctx, p->ucat_t_dev);
     delete p;
     return NBL_OK;
 }
 
-int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_dev, float *cell_dev,
-                 unsigned T, unsigned B) {
-    if(!ctx) return NBL_EINVAL;
-    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_lstm_fwd: NULL argument");
+// x_dev: dense input rows, or NULL with tokens_dev: one token per row (one-hot input)
+static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, const unsigned *tokens_dev, float *y_dev,
+                        float *cell_dev, unsigned T, unsigned B) {
     if(T == 0 || B == 0) return NBL_OK;
     const unsigned Np = 4 * p->Hp;
-    if((size_t)T * B * Np >= (1ull << 31) || (size_t)T * B * p->I >= (1ull << 31))
+    if((size_t)T * B * Np >= (1ull << 31) || (x_dev && (size_t)T * B * p->I >= (1ull << 31)))
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_lstm_fwd: tensors of 2^31 elements or more are not supported");
     int rc;
     const size_t gx_need = (size_t)T * B * Np * sizeof(float), st_need = (size_t)B * p->H * sizeof(float);
@@ -575,8 +608,18 @@ int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_de
     if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK)
         return rc;
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
-    if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
-                       p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
+    if(tokens_dev) {
+        if(!p->ucat_t_dev) {
+            if((rc = nbl_malloc(ctx, (void**)&p->ucat_t_dev, (size_t)Np * p->I * sizeof(float))) != NBL_OK) return rc;
+            hipLaunchKernelGGL(transpose_kernel, dim3(nbl_div_up(p->I, 32), nbl_div_up(Np, 32)), dim3(256), 0, ctx->stream,
+                               p->ucat_dev, p->ucat_t_dev, Np, p->I);
+            NBL_LAUNCH_CHECK(ctx, "transpose_kernel");
+        }
+        hipLaunchKernelGGL(lstm_token_gather_kernel, dim3(T * B), dim3(256), 0, ctx->stream,
+                           p->ucat_t_dev, tokens_dev, p->bu_dev, p->gx_dev, Np, p->I, p->sub_act);
+        NBL_LAUNCH_CHECK(ctx, "lstm_token_gather_kernel");
+    } else if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
+                              p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
     const size_t step = (size_t)B * p->H;
     if(p->G == 8) {
         // Recurrent half, one launch per step (lstm_step_kernel).  h_{t-1} is read straight from y[t-1].
@@ -640,6 +683,20 @@ int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_de
     if(cell_dev)
         NBL_HIP(ctx, hipMemcpyAsync(cell_dev, p->c_dev, st_need, hipMemcpyDeviceToDevice, ctx->stream));
     return NBL_OK;
+}
+
+int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, float *y_dev, float *cell_dev,
+                 unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_lstm_fwd: NULL argument");
+    return lstm_forward(ctx, p, x_dev, NULL, y_dev, cell_dev, T, B);
+}
+
+int nbl_lstm_fwd_tokens(nbl_ctx *ctx, nbl_lstm_plan *p, const unsigned *tokens_dev, float *y_dev, float *cell_dev,
+                        unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && tokens_dev && y_dev, "nbl_lstm_fwd_tokens: NULL argument");
+    return lstm_forward(ctx, p, NULL, tokens_dev, y_dev, cell_dev, T, B);
 }
 
 }  // extern "C"

@@ -345,6 +345,28 @@ static void linear_taps(unsigned dst_n, unsigned src_n, bool clamp_weight, std::
     }
 }
 
+
+// sum over rows of probs[row][target[row]] (rows whose target is outside [0, n) add nothing): what the
+// recurrent driver accumulates as  sum_i label[i] * output[i]  with one-hot labels
+// (models/networks/recurrent.cc:239-241).  One block; per-thread partial sums in row order, then a
+// fixed tree, so the result does not depend on scheduling.
+__global__ __launch_bounds__(1024) void target_prob_sum_kernel(const float *__restrict__ probs, const unsigned *__restrict__ targets,
+                                                               unsigned rows, unsigned n, float *__restrict__ out) {
+    __shared__ float red[1024];
+    float s = 0.0f;
+    for(unsigned r = threadIdx.x; r < rows; r += 1024) {
+        const unsigned t = targets[r];
+        if(t < n) s += probs[(size_t)r * n + t];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for(unsigned width = 512; width >= 1; width >>= 1) {
+        if(threadIdx.x < width) red[threadIdx.x] += red[threadIdx.x + width];
+        __syncthreads();
+    }
+    if(threadIdx.x == 0) *out = red[0];
+}
+
 }  // namespace
 
 extern "C" {
@@ -522,6 +544,15 @@ int nbl_image_to_input(nbl_ctx *ctx, const unsigned char *src_dev, unsigned imag
     hipLaunchKernelGGL(image_to_input_kernel, dim3(nbl_div_up(dst_w, 256), dst_h, images), dim3(256), 0, ctx->stream,
                        src_dev, dst_dev, ctx->rz_tab_dev, images, (int)src_h, (int)src_w, (int)channels, (int)dst_h, (int)dst_w, resize);
     NBL_LAUNCH_CHECK(ctx, "image_to_input_kernel");
+    return NBL_OK;
+}
+
+int nbl_target_prob_sum(nbl_ctx *ctx, const float *probs_dev, const unsigned *targets_dev, unsigned rows, unsigned n,
+                        float *sum_dev) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, probs_dev && targets_dev && sum_dev, "nbl_target_prob_sum: NULL pointer");
+    hipLaunchKernelGGL(target_prob_sum_kernel, dim3(1), dim3(1024), 0, ctx->stream, probs_dev, targets_dev, rows, n, sum_dev);
+    NBL_LAUNCH_CHECK(ctx, "target_prob_sum_kernel");
     return NBL_OK;
 }
 

@@ -37,6 +37,8 @@ SIGNATURES = {
     "nbl_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
     "nbl_copy_d2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_sync": (C.c_int, [_vp]),
+    "nbl_lstm_fwd_tokens": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
+    "nbl_target_prob_sum": (C.c_int, [_vp, _vp, _vp, _u, _u, _vp]),
     "nbl_image_to_input": (C.c_int, [_vp, _vp, _u, _u, _u, _u, _vp, _u, _u]),
     "nbl_conv2d_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, _u, _u, _u, _u, _u, C.c_int,
                                   C.POINTER(_vp)]),
@@ -185,6 +187,15 @@ class Ctx:
 
     def sync(self):
         self.check(lib().nbl_sync(self.h))
+
+    def target_prob_sum(self, probs, targets):
+        """sum_r probs[r][targets[r]] (probs: DeviceArray [rows][n] float32, targets: DeviceArray [rows] uint32)."""
+        rows, n = probs.shape
+        out = self.empty((1,))
+        self.check(lib().nbl_target_prob_sum(self.h, probs.ptr, targets.ptr, rows, n, out.ptr))
+        v = float(out.numpy()[0])
+        out.free()
+        return v
 
     def image_to_input(self, images_u8, dst_h, dst_w):
         """images_u8: DeviceArray [n][h][w][c] of uint8 -> DeviceArray [n][c][dst_h][dst_w] of float32."""
@@ -346,4 +357,12 @@ class LstmPlan:
         assert I == self.I
         y = out if out is not None else self.ctx.empty((T, B, self.H))
         self.ctx.check(lib().nbl_lstm_fwd(self.ctx.h, self.p, x.ptr, y.ptr, cell.ptr if cell is not None else None, T, B))
+        return y
+
+    def from_tokens(self, tokens, out=None, cell=None):
+        """tokens: DeviceArray [T][B] of uint32, the positions of the 1s of one-hot input rows."""
+        T, B = tokens.shape
+        y = out if out is not None else self.ctx.empty((T, B, self.H))
+        self.ctx.check(lib().nbl_lstm_fwd_tokens(self.ctx.h, self.p, tokens.ptr, y.ptr,
+                                                 cell.ptr if cell is not None else None, T, B))
         return y

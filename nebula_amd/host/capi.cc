@@ -122,6 +122,16 @@ int nbl_net_set_input_images(nbl_net *n, const unsigned char *host, unsigned ima
     NBL_NET_TRY(if(!n || !host) throw std::runtime_error("NULL argument"); n->net->set_input_images(host, images, height, width));
 }
 
+int nbl_net_set_input_tokens(nbl_net *n, const unsigned *host, size_t count) {
+    NBL_NET_TRY(if(!n || !host) throw std::runtime_error("NULL argument"); n->net->set_input_tokens(host, count));
+}
+
+int nbl_net_accumulate_perplexity(nbl_net *n, const unsigned *label_tokens, size_t count, float *perplexity) {
+    NBL_NET_TRY(
+        if(!n || !label_tokens || !perplexity) throw std::runtime_error("NULL argument");
+        *perplexity = n->net->accumulate_perplexity(label_tokens, count));
+}
+
 int nbl_net_forward(nbl_net *n) {
     NBL_NET_TRY(if(!n) throw std::runtime_error("NULL argument"); n->net->forward());
 }

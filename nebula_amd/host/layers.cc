@@ -511,6 +511,13 @@ void lstm_layer_t::pack() {
 // network->batch_size counts every (time step, sequence) row; rows are time-major.
 void lstm_layer_t::_forward_() {
     if(!plan) throw std::runtime_error("Error: lstm layer has no weights (init_weight not called)");
+    if(!prev_layer && network->input_tokens_dev) {      // one-hot input rows given as token indices
+        nbl_check(network->ctx,
+                  nbl_lstm_fwd_tokens(network->ctx, plan, network->input_tokens_dev, output_data_dev, NULL,
+                                      network->time_step, network->batch_size / network->time_step),
+                  "nbl_lstm_fwd_tokens");
+        return;
+    }
     nbl_check(network->ctx,
               nbl_lstm_fwd(network->ctx, plan, input_dev(), output_data_dev, NULL,
                            network->time_step, network->batch_size / network->time_step),

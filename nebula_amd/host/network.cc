@@ -1,5 +1,7 @@
 #include "network.h"
 
+#include <cmath>
+
 #include <hip/hip_runtime_api.h>
 
 #include <fstream>
@@ -22,7 +24,7 @@ network_t::network_t() :
     run_type(UNDEFINED_RUN), num_threads(1),
     learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
     input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
-    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), conv_split(-1),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1),
     input_layer(NULL), output_layer(NULL), num_layers(0) {}
 
 network_t::~network_t() {}
@@ -65,7 +67,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
     last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false),
-    image_staging_dev(NULL), image_staging_bytes(0) {
+    cumulative_cost(0.0f), rows_seen(0), image_staging_dev(NULL), image_staging_bytes(0), tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
@@ -81,6 +83,7 @@ inference_net_t::~inference_net_t() {
     for(size_t i = 0; i < events.size(); i++) (void)hipEventDestroy((hipEvent_t)events[i]);
     if(input_data_dev && ctx) nbl_free(ctx, input_data_dev);
     if(image_staging_dev && ctx) nbl_free(ctx, image_staging_dev);
+    if(ctx) { nbl_free(ctx, tokens_dev); nbl_free(ctx, labels_dev); nbl_free(ctx, cost_dev); }
     delete [] input_data;
     if(ctx) nbl_ctx_destroy(ctx);
 }
@@ -172,6 +175,36 @@ void inference_net_t::set_input(const float *host, size_t count) {
     if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     if(count != (size_t)batch_size * input_size) throw std::runtime_error("Error: input tensor has the wrong size");
     nbl_check(ctx, nbl_h2d(ctx, input_data_dev, host, count * sizeof(float)), "nbl_h2d(input)");
+    input_tokens_dev = NULL;
+}
+
+void inference_net_t::set_input_tokens(const unsigned *host, size_t count) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
+    if(!is_recurrent) throw std::runtime_error("Error: token input on a network without time_steps");
+    if(count != (size_t)batch_size) throw std::runtime_error("Error: token input has the wrong size");
+    if(layers.empty() || layers[0]->layer_type != LSTM_LAYER)
+        throw std::runtime_error("Error: token input needs an lstm layer first");
+    if(!tokens_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&tokens_dev, (size_t)batch_size * sizeof(unsigned)), "nbl_malloc(tokens)");
+    nbl_check(ctx, nbl_h2d(ctx, tokens_dev, host, count * sizeof(unsigned)), "nbl_h2d(tokens)");
+    input_tokens_dev = tokens_dev;
+}
+
+float inference_net_t::accumulate_perplexity(const unsigned *label_tokens_host, size_t count) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
+    if(!output_layer) throw std::runtime_error("Error: network has no layers");
+    // rows the output layer holds: every (time step, sequence) row, or the last step's with last_step_only
+    const size_t rows = last_step_only && is_recurrent ? batch_size / time_step : batch_size;
+    if(count != rows) throw std::runtime_error("Error: label tokens have the wrong size");
+    if(!labels_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&labels_dev, (size_t)batch_size * sizeof(unsigned)), "nbl_malloc(labels)");
+    if(!cost_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&cost_dev, 16), "nbl_malloc(cost)");
+    nbl_check(ctx, nbl_h2d(ctx, labels_dev, label_tokens_host, count * sizeof(unsigned)), "nbl_h2d(labels)");
+    nbl_check(ctx, nbl_target_prob_sum(ctx, output_layer->output_data_dev, labels_dev, (unsigned)rows, output_layer->output_size,
+                                       cost_dev), "nbl_target_prob_sum");
+    float sum = 0.0f;
+    nbl_check(ctx, nbl_d2h(ctx, &sum, cost_dev, sizeof(float)), "nbl_d2h(cost)");
+    cumulative_cost += sum;
+    rows_seen += rows;
+    return std::exp(-1.0f * std::log2(cumulative_cost / (float)rows_seen));
 }
 
 // The image driver's load_data() contract (models/networks/convolutional.cc:384-412) with the resize,

@@ -47,6 +47,9 @@ public:
     float *input_data_dev;              // device input [batch_size][input_size]
 
     nbl_ctx *ctx;                       // takes the place of cublas_handle / cudnn_handle
+    // Recurrent nets fed by set_input_tokens(): position of the 1 in each one-hot input row, [T*B] time-major
+    // (NULL while the dense input_data_dev is the input).  The first layer, if an LSTM, gathers instead of multiplying.
+    unsigned *input_tokens_dev;
     // [net] key `conv_split` (a key the reference ignores): 0 = convolutions never split their sum over
     // the patch rows between blocks, 1 = wherever the cost model says so; absent = measured per layer on
     // first use.  With 0 a convolution's result does not depend on the tile shape the search picks.
@@ -81,6 +84,13 @@ public:
     // `images` 8-bit interleaved images [height][width][input_channel] (channel order B, G, R as decoded) ->
     // network input, as convolutional_t::load_data() prepares it (resize, / 255, planes 0 and 2 swapped).
     void set_input_images(const unsigned char *host, unsigned images, unsigned height, unsigned width);
+    // The recurrent driver's load_data() (models/networks/recurrent.cc:179-204) without materialising the one-hot
+    // matrix: tokens[T*B] time-major, each the index of the 1.0 of its input row.  A later set_input() switches back.
+    void set_input_tokens(const unsigned *host, size_t count);
+    // recurrent_t::print_results(), test branch (recurrent.cc:239-247): adds sum_rows probability(label token) of
+    // the output layer to cumulative_cost and returns exp(-log2(cumulative_cost / rows seen so far)).
+    float accumulate_perplexity(const unsigned *label_tokens_host, size_t count);
+    float cumulative_cost; size_t rows_seen;
     void run(const std::string m_output_weight = "");
     bool recurrent() const { return is_recurrent; }
 
@@ -110,6 +120,7 @@ private:
     unsigned batch_override;
     bool is_recurrent;
     unsigned char *image_staging_dev;   // device copy of the last byte-image batch
+    unsigned *tokens_dev, *labels_dev; float *cost_dev;   // token input, label tokens and the device-side sum
     size_t image_staging_bytes;
     std::vector<void*> events;
 };

@@ -27,6 +27,8 @@ SIGNATURES = {
     "nbl_net_layer_flop": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),
     "nbl_net_set_input": (C.c_int, [_vp, _vp, C.c_size_t]),
     "nbl_net_set_input_images": (C.c_int, [_vp, _vp, _u, _u, _u]),
+    "nbl_net_set_input_tokens": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "nbl_net_accumulate_perplexity": (C.c_int, [_vp, _vp, C.c_size_t, C.POINTER(C.c_float)]),
     "nbl_net_forward": (C.c_int, [_vp]),
     "nbl_net_sync": (C.c_int, [_vp]),
     "nbl_net_forward_timed": (C.c_int, [_vp, C.POINTER(C.c_float)]),
@@ -133,6 +135,17 @@ class Network:
         a = np.ascontiguousarray(images_u8, np.uint8)
         n, h, w, _ = a.shape
         self._check(lib().nbl_net_set_input_images(self.h, a.ctypes.data, n, h, w))
+
+    def set_input_tokens(self, tokens):
+        """uint32 [time_steps][sequences]: index of the 1 of every one-hot input row."""
+        t = np.ascontiguousarray(tokens, np.uint32)
+        self._check(lib().nbl_net_set_input_tokens(self.h, t.ctypes.data, t.size))
+
+    def accumulate_perplexity(self, label_tokens):
+        t = np.ascontiguousarray(label_tokens, np.uint32)
+        out = C.c_float()
+        self._check(lib().nbl_net_accumulate_perplexity(self.h, t.ctypes.data, t.size, C.byref(out)))
+        return out.value
 
     def forward(self):
         self._check(lib().nbl_net_forward(self.h))

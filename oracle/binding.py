@@ -89,6 +89,10 @@ def oracle():
         lib.orc_avgpool_forward.argtypes = [_f32p, _f32p] + [_u] * 7
         lib.orc_shortcut_forward.argtypes = [_f32p, _f32p, _f32p] + [_u] * 8
         lib.orc_softmax_forward.argtypes = [_f32p, _f32p, _u, _u]
+        lib.orc_target_prob_sum.argtypes = [_f32p, C.c_void_p, _u, _u]
+        lib.orc_target_prob_sum.restype = C.c_float
+        lib.orc_perplexity.argtypes = [C.c_float, _u]
+        lib.orc_perplexity.restype = C.c_float
         lib.orc_image_to_input.argtypes = [C.c_void_p, _u, _u, _u, _f32p, _u, _u]
         lib.orc_resize_linear_u8.argtypes = [C.c_void_p, _u, _u, _u, C.c_void_p, _u, _u]
         pp = C.POINTER(_f32p)
@@ -217,6 +221,16 @@ def shortcut_forward(prev, conn, act="linear"):
     out = np.empty_like(prev)
     oracle().orc_shortcut_forward(_fp(prev), _fp(conn), _fp(out), B, ic, ih, iw, oc, oh, ow, ACT[act])
     return out
+
+
+def target_prob_sum(probs, targets):
+    probs = _f32(probs); targets = np.ascontiguousarray(targets, np.uint32)
+    rows, n = probs.shape
+    return float(oracle().orc_target_prob_sum(_fp(probs), targets.ctypes.data, rows, n))
+
+
+def perplexity(cumulative_cost, rows_seen):
+    return float(oracle().orc_perplexity(cumulative_cost, rows_seen))
 
 
 def image_to_input(img, dst_h, dst_w):

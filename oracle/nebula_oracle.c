@@ -460,6 +460,21 @@ void orc_image_to_input(const unsigned char *src, unsigned src_h, unsigned src_w
     free(tmp);
 }
 
+/* recurrent_t::print_results(), test branch (models/networks/recurrent.cc:239-247) with the one-hot labels
+ * of load_data (:193-197): cumulative_cost += label[i] * output[i] over every element in order (float;
+ * the zero labels add +0), then the printed figure exp(-log2(cumulative_cost / rows_seen)), evaluated in
+ * float as the C++ overloads do for float arguments. */
+float orc_target_prob_sum(const float *probs, const unsigned *targets, unsigned rows, unsigned n) {
+    float cum = 0.0f;
+    for(unsigned r = 0; r < rows; r++)
+        for(unsigned j = 0; j < n; j++) cum += (targets[r] == j ? 1.0f : 0.0f) * probs[(size_t)r * n + j];
+    return cum;
+}
+
+float orc_perplexity(float cumulative_cost, unsigned rows_seen) {
+    return expf(-1.0f * log2f(cumulative_cost / (float)rows_seen));
+}
+
 /* ---------------------------------------------------------------------------------------
  * LSTM, lstm_layer.cc:233-346.  Sub-layer slots in file order (lstm_layer.cc:194-206):
  *   0 iW  1 fW  2 oW  3 cW  4 iU  5 fU  6 oU  7 cU

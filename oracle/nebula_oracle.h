@@ -93,6 +93,11 @@ void orc_shortcut_forward(const float *prev, const float *conn, float *out, unsi
 /* models/layers/softmax_layer.cc:85-106 */
 void orc_softmax_forward(const float *x, float *y, unsigned rows, unsigned n);
 
+/* recurrent_t::print_results() (models/networks/recurrent.cc:239-247): sum of label * output with one-hot
+ * labels, and the "perplexity" figure the driver prints from it. */
+float orc_target_prob_sum(const float *probs, const unsigned *targets, unsigned rows, unsigned n);
+float orc_perplexity(float cumulative_cost, unsigned rows_seen);
+
 /* convolutional_t::load_data (models/networks/convolutional.cc:384-412): 8-bit interleaved image ->
  * network input planes (resize if needed, / 255.0, planes 0 and 2 swapped).  The resize restates
  * OpenCV's 8-bit INTER_LINEAR and is PARITY UNPINNED (OpenCV is absent; see the .c file). */

@@ -271,3 +271,43 @@ def test_network_input_from_byte_images():
         b = [net.output(i) for i in range(net.num_layers)]
     for u, v in zip(a, b):
         np.testing.assert_array_equal(u.view(np.uint32), v.view(np.uint32))
+
+
+def test_recurrent_driver_contract_tokens_and_perplexity():
+    """Token input == one-hot input through the whole network; the perplexity figure follows recurrent.cc:239-247."""
+    from nebula_amd import zoo
+    from nebula_amd.net import Network
+    print("CASE recurrent tokens + perplexity", flush=True)
+    T, B, V, H = 6, 5, 40, 128
+    rng = np.random.default_rng(31)
+    cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=2, classes=V)
+    onet = ob.OracleNet(cfg)
+    blob = np.concatenate([rng.uniform(-1, 1, int(np.prod(sh))).astype(np.float32) / np.float32(np.sqrt(H))
+                           for _, _, sh in ob.weight_layout(onet.specs)])
+    onet.load_weights(blob)
+    tokens = rng.integers(0, V, (T, B)).astype(np.uint32)
+    labels = rng.integers(0, V, (T, B)).astype(np.uint32)
+    x = np.zeros((T, B, V), np.float32)
+    x[np.arange(T)[:, None], np.arange(B)[None, :], tokens] = 1.0
+    ob.use_custom_gemm()
+    want = onet.forward(x)
+    probs_want = want[-1].reshape(T * B, V)
+    with Network(cfg) as net:
+        net.load_weight_blob(blob)
+        net.set_input(x)
+        net.forward()
+        dense = [net.output(i) for i in range(net.num_layers)]
+        net.set_input_tokens(tokens)
+        net.forward()
+        tok = [net.output(i) for i in range(net.num_layers)]
+        for u, v in zip(dense, tok):
+            np.testing.assert_array_equal(u.view(np.uint32), v.view(np.uint32))
+        assert rel(tok[-1], probs_want.ravel()) <= TOL
+        cum = 0.0
+        for it in range(2):                      # two "iterations" of the driver on the same batch
+            got = net.accumulate_perplexity(labels)
+            cum = np.float32(cum + ob.target_prob_sum(probs_want, labels.ravel()))
+            assert abs(got - ob.perplexity(float(cum), (it + 1) * T * B)) <= 1e-4 * got
+        net.set_input(x)                          # back to the dense input
+        net.forward()
+        np.testing.assert_array_equal(net.output(0).view(np.uint32), dense[0].view(np.uint32))

@@ -371,6 +371,43 @@ def test_lstm_matches_oracle(ctx, case):
     np.testing.assert_array_equal(bits(got2), bits(got))
 
 
+@pytest.mark.parametrize("H", [128, 33])
+def test_lstm_token_input_equals_one_hot_input(ctx, H):
+    """One-hot input rows given as token indices: the gather must reproduce the dense product bit for bit."""
+    announce("lstm tokens", H)
+    T, B, V = 5, 7, 50
+    rng = np.random.default_rng(H)
+    tokens = rng.integers(0, V, (T, B)).astype(np.uint32)
+    tokens[2, 3] = V + 5                                  # outside the vocabulary: an all-zero input row
+    x = np.zeros((T, B, V), np.float32)
+    for t in range(T):
+        for b in range(B):
+            if tokens[t, b] < V:
+                x[t, b, tokens[t, b]] = 1.0
+    names = ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU")
+    wt = [(rng.uniform(-1, 1, (H, H if n[1] == "W" else V)) / np.sqrt(H)).astype(np.float32) for n in names]
+    bs = [(rng.uniform(-1, 1, H) / np.sqrt(H)).astype(np.float32) for n in names]
+    want = ob.lstm_forward(x, wt, bs, None, "linear")
+    plan = ctx.lstm_pack(wt, bs, None, "linear")
+    dense = plan(ctx.array(x)).numpy()
+    got = plan.from_tokens(ctx.array(tokens, dtype=np.uint32)).numpy()
+    np.testing.assert_array_equal(bits(got), bits(dense))
+    assert rel(got, want) <= TOL
+
+
+def test_target_prob_sum_and_perplexity(ctx):
+    announce("target prob sum")
+    rng = np.random.default_rng(77)
+    for rows, n in ((1, 5), (37, 11), (4096, 1000)):
+        p = rng.random((rows, n), dtype=np.float32)
+        p /= p.sum(1, keepdims=True)
+        t = rng.integers(0, n, rows).astype(np.uint32)
+        want = ob.target_prob_sum(p, t)
+        got = ctx.target_prob_sum(ctx.array(p), ctx.array(t, dtype=np.uint32))
+        assert abs(got - want) <= 1e-5 * abs(want), (rows, n, got, want)
+        assert abs(got - float(p[np.arange(rows), t].astype(np.float64).sum())) <= 1e-5 * abs(want)
+
+
 def test_error_paths(ctx):
     from nebula_amd import hip
     import ctypes as C
