@@ -68,6 +68,10 @@ def workload(name, batch):
         "conv1": (zoo.conv1_pool_cfg, 32, "uniform", "he", "AlexNet conv1+ReLU+maxpool fp32, batch %d"),
         "lstm": (lambda b: zoo.lstm_cfg(b, last_step_only=True), 64, "normal", "lstm",
                  "2-layer LSTM 1024/1024 T=64 + 10000-way projection and softmax on the last step, batch %d"),
+        "rnn": (zoo.rnn_cfg, 32, "normal", "he",
+                "rnn_large: 5 normalised RNN layers of 1024, T=40, 8713-way projection and softmax on every step, batch %d"),
+        "dbn": (zoo.dbn_cfg, 32, "uniform", "he", "dbn_large: 4 RBM layers + 62-way classifier on 3x128x128 U[0,1), batch %d"),
+        "mlp": (zoo.mlp_cfg, 32, "uniform", "he", "mlp_large: 5 relu layers + 62-way classifier on 3x128x128 U[0,1), batch %d"),
     }
     fn, default_batch, xdist, wdist, text = table[name]
     b = batch or default_batch
@@ -218,7 +222,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "copy", "conv", "images", "ptb"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "images", "ptb"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
                          "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
                          "for counter passes over a single kernel")
@@ -245,7 +249,7 @@ def main():
     from nebula_amd.net import Network
 
     cfg, batch, xdist, wdist, text = workload(args.workload, args.batch)
-    is_lstm = args.workload == "lstm"
+    is_lstm = args.workload in ("lstm", "rnn")        # recurrent: units are sequences, rows are time steps x sequences
     rng = np.random.default_rng(20240611)
     net = Network(cfg)
     blob = make_weights(net.weight_layout(), rng, wdist)
@@ -289,14 +293,27 @@ def main():
     log("per-layer-kind ms:", {k: round(v, 3) for k, v in by_kind.items()})
     algo_bytes = 0.0
     fused = "fuse_shortcut=1" in cfg
+    roofline = None
     if is_lstm:
-        # 2*B*(I+H)*4H per step per layer
-        lstm_flop = sum(2.0 * net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])
-                        * 4 * net.layer_info(i)["output_size"] for i, k in enumerate(kinds) if k == "lstm_layer")
-        dom_ms = by_kind.get("lstm_layer", 0.0)
-        n_launch = sum(k == "lstm_layer" for k in kinds)
-        achieved = lstm_flop / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
-        dom_name = "lstm (input GEMM + fused recurrent steps)"
+        # per row: 2*(I+H)*4H (lstm), 2*(I+2*O)*O (rnn)
+        rec = [i for i, k in enumerate(kinds) if k in ("lstm_layer", "rnn_layer")]
+        dom_ms = float(layer_ms[rec].sum())
+        n_launch = len(rec)
+        achieved = float(flops[rec].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
+        dom_name = "%s layers (input product over all steps + one fused kernel per time step)" % args.workload
+    elif args.workload in ("dbn", "mlp"):
+        # weight streaming: every layer reads its [O][I] matrix once per step
+        fc = [i for i, k in enumerate(kinds) if k in ("connected_layer", "rbm_layer")]
+        dom_ms = float(layer_ms[fc].sum())
+        n_launch = len(fc)
+        fc_bytes = sum(4.0 * (net.layer_info(i)["input_size"] * net.layer_info(i)["output_size"]
+                              + net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])) for i in fc)
+        gbps = fc_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+        roofline = {"bound": "hbm", "kernel": "gemm_nt_kernel (split-K) + splitk_reduce_kernel", "achieved": round(gbps, 1),
+                    "peak": 8000.0, "unit": "GB/s", "frac": round(gbps / 8000.0, 4), "traffic": None,
+                    "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4),
+                    "algorithmic_bytes_per_launch": round(fc_bytes / max(n_launch, 1)),
+                    "tflops": round(float(flops[fc].sum()) / (dom_ms * 1e-3) / 1e12, 2) if dom_ms > 0 else 0.0}
     else:
         conv = [i for i, k in enumerate(kinds) if k == "convolutional_layer"]
         dom_ms = float(layer_ms[conv].sum())
@@ -309,10 +326,11 @@ def main():
             weights = net.layer_flop(i) / (2.0 * info["output_height"] * info["output_width"])
             residual = info["output_size"] if i + 1 < len(kinds) and kinds[i + 1] == "shortcut_layer" and fused else 0
             algo_bytes += 4.0 * (net.batch_size * (info["input_size"] + info["output_size"] + residual) + weights)
-    roofline = {"bound": "mfma", "kernel": dom_name, "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, batch)),
-                "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4)}
+    if roofline is None:
+        roofline = {"bound": "mfma", "kernel": dom_name, "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, batch)),
+                    "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4)}
     if algo_bytes:
         roofline["algorithmic_bytes_per_launch"] = round(algo_bytes / n_launch)
         roofline["algorithmic_flop_per_launch"] = round(float(flops[conv].sum()) / n_launch)
@@ -329,7 +347,7 @@ def main():
 
     if not args.no_cpu and args.cpu_sample != 0:
         from nebula_amd import zoo
-        sample = args.cpu_sample if args.cpu_sample > 0 else {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4}[args.workload]
+        sample = args.cpu_sample if args.cpu_sample > 0 else {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4, "rnn": 4, "dbn": 32, "mlp": 32}[args.workload]
         cfg_fn = (lambda b: workload(args.workload, b)[0])
         ips, cores, dt, blas, xs, outs = cpu_baseline(cfg_fn, blob, xdist, sample, is_lstm, np.random.default_rng(7))
         result["cpu_baseline"] = {"value": round(ips, 3), "unit": result["unit"], "cores": cores, "kind": "port",

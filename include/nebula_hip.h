@@ -28,6 +28,7 @@ typedef struct nbl_ctx nbl_ctx;
 typedef struct nbl_conv_plan nbl_conv_plan;
 typedef struct nbl_fc_plan nbl_fc_plan;
 typedef struct nbl_lstm_plan nbl_lstm_plan;
+typedef struct nbl_rnn_plan nbl_rnn_plan;
 
 enum nbl_status {
     NBL_OK = 0,
@@ -169,6 +170,28 @@ int nbl_lstm_fwd_tokens(nbl_ctx *ctx, nbl_lstm_plan *plan, const unsigned *token
 int nbl_target_prob_sum(nbl_ctx *ctx, const float *probs_dev, const unsigned *targets_dev, unsigned rows, unsigned n,
                         float *sum_dev);
 int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *plan);
+
+/* ---- RNN layer ---------------------------------------------------------------------------------
+ * nbl_rnn_pack: rnn_layer_t::init_weight() (models/layers/rnn_layer.cc:73-77): three connected sub-layers as
+ * HOST arrays in FILE order input gate [O][I], hidden gate [O][O], output gate [O][O] (bias [O] each;
+ * scale/mean/var: three [O] vectors each, or NULL when batch_normalize=0); act is the [rnn] section's
+ * activation, applied inside every sub-layer.
+ * nbl_rnn_fwd: rnn_layer_t::forward() (rnn_layer.cc:91-141): x_dev [T][B][I] -> y_dev [T][B][O],
+ *   in_t = input(x_t);  hid_t = hidden(t == 0 ? in_0 : state_{t-1});  state_t = in_t + hid_t;
+ *   y_t = output(t == 0 ? hid_0 : state_t)
+ * (step 0 reads the neighbouring sub-layers as the reference does).  The input gate of all steps is one
+ * product, the recurrence one fused kernel per step, the output gate of steps 1..T-1 one product. */
+int nbl_rnn_pack(nbl_ctx *ctx, const float *const *weight_host, const float *const *bias_host,
+                 const float *const *scale_host, const float *const *mean_host, const float *const *var_host,
+                 unsigned I, unsigned O, int act, nbl_rnn_plan **out);
+int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *plan, const float *x_dev, float *y_dev, unsigned T, unsigned B);
+int nbl_rnn_plan_destroy(nbl_ctx *ctx, nbl_rnn_plan *plan);
+
+/* count_dev[0] = number of rows whose label is among the k largest entries of probs[row][0..n): the
+ * matches convolutional_t::print_results() counts (models/networks/convolutional.cc:428-447).  Equal
+ * entries rank by ascending class index (the reference's std::sort leaves their order open). */
+int nbl_topk_matches(nbl_ctx *ctx, const float *probs_dev, const unsigned *labels_dev, unsigned rows, unsigned n,
+                     unsigned k, unsigned *count_dev);
 
 /* ---- memory-bound layers -----------------------------------------------------------------------
  * nbl_pool_fwd: pooling_layer_t::_forward_() (models/layers/pooling_layer.cu:150-172; CPU twin

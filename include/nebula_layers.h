@@ -42,7 +42,8 @@ int nbl_net_num_layers(nbl_net *net);
 /* info[0..7] = layer_type, activation_type, output_channel, output_height, output_width, output_size,
  * input_size, padding */
 int nbl_net_layer_info(nbl_net *net, int layer, unsigned *info);
-/* 2*F*OH*OW*C*k*k for a convolutional layer, 2*I*O for a connected one, 0 otherwise (per input row) */
+/* per input row: 2*F*OH*OW*C*k*k for a convolutional layer, 2*I*O for a connected / rbm one, 2*(I+2*O)*O for an
+ * rnn layer, 2*(I+H)*4H for an lstm layer, 0 otherwise */
 int nbl_net_layer_flop(nbl_net *net, int layer, double *flop_per_row);
 /* host -> device input, [batch_size][input_size] floats */
 int nbl_net_set_input(nbl_net *net, const float *host, size_t count);
@@ -59,6 +60,10 @@ int nbl_net_set_input_tokens(nbl_net *net, const unsigned *host, size_t count);
  * probabilities of the label tokens (one per output row) to the running sum and returns the driver's figure
  * exp(-log2(sum / rows seen)). */
 int nbl_net_accumulate_perplexity(nbl_net *net, const unsigned *label_tokens, size_t count, float *perplexity);
+/* convolutional_t::print_results(), test branch (models/networks/convolutional.cc:428-447): after a forward,
+ * adds the number of rows whose label is among the output layer's k largest entries to a running count of
+ * matches and returns that count (the reference's static `matches`).  labels: one class index per output row. */
+int nbl_net_accumulate_topk(nbl_net *net, const unsigned *labels, size_t count, unsigned k, unsigned *matches);
 /* network_t::forward(); asynchronous unless the net ends in a softmax (which copies to the host) */
 int nbl_net_forward(nbl_net *net);
 int nbl_net_sync(nbl_net *net);

@@ -227,35 +227,16 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__re
     y[e] = nbl_act_apply(act, v);
 }
 
-// One LSTM time step in one launch, for layers packed with gate interleave 8 (row of gate g, hidden unit
-// h: (h/8)*32 + g*8 + h%8), so that ONE 32x32 MFMA tile holds the four gate pre-activations of 8 hidden
-// units for 32 batch rows.  A step is latency, not throughput ([B x H].[H x 4H] is 3.4 us of MFMA time
-// on the whole chip), so the work is cut for many small independent pieces: a block owns one such
-// tile, its four waves each take a quarter of the k range and read their MFMA operands STRAIGHT from
-// global memory (each lane one 16-byte piece of its row per 8 k: lanes 0-31 supply k+0..3, lanes
-// 32-63 k+4..7 of both operands, which is a legal pairing), several loads in flight per lane and no
-// barrier until the four partial tiles meet in LDS.  Then each thread owns one (batch row, hidden
-// unit): sum of the four partial tiles for each gate, bias, input-side pre-activation, the cell update
-// (lstm_layer.cc:264-312, each product rounded on its own) and h_t written into y[t], which is the
-// next step's operand.  Needs H % 128 == 0 and 16-byte aligned rows.
-struct LstmStepArgs {
-    const float *hprev; const float *w; const float *gx; const float *bw; float *c; float *hout;
-    int B, H, Np, sub_act;
-};
-
-__global__ __launch_bounds__(256)
-void lstm_step_kernel(const LstmStepArgs a) {
+// A wave's share of a skinny product: acc0 + acc1 = sum over `kw` consecutive k of A[row][k] * B[col][k]
+// as one 32x32 MFMA tile, with both operands read STRAIGHT from global memory: ap / bp point at the
+// lane's row (lane % 32) of each operand, advanced by 4 floats for lanes 32-63, so that per 8 k the
+// lanes 0-31 supply k+0..3 and lanes 32-63 k+4..7 of both operands (a legal pairing).  Loads run one
+// batch of U steps ahead; two accumulators take turns because with one wave per SIMD nothing else
+// hides the latency between two MFMAs on the same registers.  kw must be a multiple of 32.
+__device__ __forceinline__ void wave_tile_from_global(const float *__restrict__ ap, const float *__restrict__ bp, int kw,
+                                                      floatx16 &acc0, floatx16 &acc1) {
     constexpr int U = 4;                    // 8-wide k steps per batch of loads
-    __shared__ float red[4][32][33];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 31, half = lane >> 5;
-    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
-    const int kw = a.H >> 2;                // k range of one wave
-    const int arow = min(m0 + r, a.B - 1);  // rows past the batch repeat the last one; their sums are dropped
-    const float *__restrict__ ap = a.hprev + (size_t)arow * a.H + wave * kw + half * 4;
-    const float *__restrict__ bp = a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4;
     const int nb = kw / (8 * U);
-
     float4 av[2][U], bv[2][U];
     auto load = [&](int buf, int b) {
         #pragma unroll
@@ -264,9 +245,6 @@ void lstm_step_kernel(const LstmStepArgs a) {
             bv[buf][u] = *reinterpret_cast<const float4*>(bp + (b * U + u) * 8);
         }
     };
-    // two accumulators take turns: with one wave per SIMD nothing else hides the latency between two
-    // MFMAs on the same registers
-    floatx16 acc0, acc1;
     #pragma unroll
     for(int i = 0; i < 16; i++) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
     auto compute = [&](int buf) {
@@ -287,6 +265,35 @@ void lstm_step_kernel(const LstmStepArgs a) {
         compute(1);
     }
     if(b < nb) compute(0);
+}
+
+// One LSTM time step in one launch, for layers packed with gate interleave 8 (row of gate g, hidden unit
+// h: (h/8)*32 + g*8 + h%8), so that ONE 32x32 MFMA tile holds the four gate pre-activations of 8 hidden
+// units for 32 batch rows.  A step is latency, not throughput ([B x H].[H x 4H] is 3.4 us of MFMA time
+// on the whole chip), so the work is cut for many small independent pieces: a block owns one such
+// tile, its four waves each take a quarter of the k range and read their MFMA operands STRAIGHT from
+// global memory (each lane one 16-byte piece of its row per 8 k: lanes 0-31 supply k+0..3, lanes
+// 32-63 k+4..7 of both operands, which is a legal pairing), several loads in flight per lane and no
+// barrier until the four partial tiles meet in LDS.  Then each thread owns one (batch row, hidden
+// unit): sum of the four partial tiles for each gate, bias, input-side pre-activation, the cell update
+// (lstm_layer.cc:264-312, each product rounded on its own) and h_t written into y[t], which is the
+// next step's operand.  Needs H % 128 == 0 and 16-byte aligned rows.
+struct LstmStepArgs {
+    const float *hprev; const float *w; const float *gx; const float *bw; float *c; float *hout;
+    int B, H, Np, sub_act;
+};
+
+__global__ __launch_bounds__(256)
+void lstm_step_kernel(const LstmStepArgs a) {
+    __shared__ float red[4][32][33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int kw = a.H >> 2;                // k range of one wave
+    const int arow = min(m0 + r, a.B - 1);  // rows past the batch repeat the last one; their sums are dropped
+    floatx16 acc0, acc1;
+    wave_tile_from_global(a.hprev + (size_t)arow * a.H + wave * kw + half * 4,
+                          a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4, kw, acc0, acc1);
 
     // accumulator register i of a 32x32 tile: row 8*(i/4) + 4*(lane/32) + i%4 (batch), column lane%32 (gate column)
     #pragma unroll
@@ -312,6 +319,53 @@ void lstm_step_kernel(const LstmStepArgs a) {
     const float ct = __fadd_rn(cf, ig);
     a.c[e] = ct;
     a.hout[e] = __fmul_rn(lstm_tanh(ct), go);
+}
+
+// One step of the RNN layer's recurrence (rnn_layer.cc:100-115) in one launch, same work split as
+// lstm_step_kernel: hid = act((prev . Wh^T) * g + b), state = in_t + hid; a block owns a 32x32 tile of
+// the [B x O] step.  hid is also stored where the caller wants it (step 0's output gate reads it).
+struct RnnStepArgs {
+    const float *prev; const float *w; const float *g; const float *b; const float *in_t;
+    float *state; float *hid;        // hid may be NULL
+    int B, H, act;                   // H = layer width (rows of Wh and its fan-in)
+};
+
+__global__ __launch_bounds__(256)
+void rnn_step_kernel(const RnnStepArgs a) {
+    __shared__ float red[4][32][33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int kw = a.H >> 2;
+    const int arow = min(m0 + r, a.B - 1);
+    floatx16 acc0, acc1;
+    wave_tile_from_global(a.prev + (size_t)arow * a.H + wave * kw + half * 4,
+                          a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4, kw, acc0, acc1);
+    #pragma unroll
+    for(int i = 0; i < 16; i++) red[wave][8 * (i >> 2) + 4 * half + (i & 3)][r] = acc0[i] + acc1[i];
+    __syncthreads();
+    // thread -> 4 adjacent columns of one row
+    const int ml = tid >> 3, c4 = (tid & 7) * 4;
+    const int m = m0 + ml;
+    if(m >= a.B) return;
+    float v[4];
+    #pragma unroll
+    for(int j = 0; j < 4; j++) {
+        const int col = c4 + j, n = n0 + col;
+        const float sum = (red[0][ml][col] + red[1][ml][col]) + (red[2][ml][col] + red[3][ml][col]);
+        v[j] = nbl_act_apply(a.act, __builtin_fmaf(sum, a.g[n], a.b[n]));
+    }
+    const size_t e = (size_t)m * a.H + n0 + c4;
+    const float4 in = *reinterpret_cast<const float4*>(a.in_t + e);
+    if(a.hid) *reinterpret_cast<float4*>(a.hid + e) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(a.state + e) = make_float4(__fadd_rn(in.x, v[0]), __fadd_rn(in.y, v[1]),
+                                                          __fadd_rn(in.z, v[2]), __fadd_rn(in.w, v[3]));
+}
+
+// state = a + b elementwise (the two axpy of rnn_layer.cc:108-115 on a zeroed state)
+__global__ void add_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(i < n) out[i] = __fadd_rn(a[i], b[i]);
 }
 
 // LSTM cell for one time step from split-K partial sums of the recurrent GEMM:
@@ -402,6 +456,14 @@ struct nbl_lstm_plan {
     float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
     float *ucat_t_dev;                    // [I][4*Hp] transpose of ucat_dev, built on the first token-input forward
     unsigned G;                           // gate interleave: row of (gate, h) = (h/G)*4G + gate*G + h%G; 8 = single-launch steps
+};
+
+// rnn_layer_t: three connected sub-layers (input, hidden, output gate) and the per-forward buffers
+struct nbl_rnn_plan {
+    unsigned I, O;
+    nbl_fc_plan *gate[3];
+    float *in_all, *states, *hid0, *tmp;     // [T*B][O], [T*B][O], [B][O], [B][O]
+    size_t rows_alloc, seqs_alloc;
 };
 
 namespace {
@@ -697,6 +759,91 @@ int nbl_lstm_fwd_tokens(nbl_ctx *ctx, nbl_lstm_plan *p, const unsigned *tokens_d
     if(!ctx) return NBL_EINVAL;
     NBL_REQUIRE(ctx, p && tokens_dev && y_dev, "nbl_lstm_fwd_tokens: NULL argument");
     return lstm_forward(ctx, p, NULL, tokens_dev, y_dev, cell_dev, T, B);
+}
+
+int nbl_rnn_pack(nbl_ctx *ctx, const float *const *weight_host, const float *const *bias_host,
+                 const float *const *scale_host, const float *const *mean_host, const float *const *var_host,
+                 unsigned I, unsigned O, int act, nbl_rnn_plan **out) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, out != NULL, "nbl_rnn_pack: out is NULL");
+    *out = NULL;
+    NBL_REQUIRE(ctx, weight_host && bias_host, "nbl_rnn_pack: weight/bias is NULL");
+    NBL_REQUIRE(ctx, (scale_host != NULL) == (mean_host != NULL) && (scale_host != NULL) == (var_host != NULL),
+                "nbl_rnn_pack: scale, mean and var must be given together");
+    NBL_REQUIRE(ctx, I && O, "nbl_rnn_pack: zero dimension");
+    nbl_rnn_plan *p = new nbl_rnn_plan();
+    memset(p, 0, sizeof(*p));
+    p->I = I; p->O = O;
+    for(int s = 0; s < 3; s++) {
+        const int rc = nbl_fc_pack(ctx, weight_host[s], bias_host[s], scale_host ? scale_host[s] : NULL,
+                                   mean_host ? mean_host[s] : NULL, var_host ? var_host[s] : NULL,
+                                   s == 0 ? I : O, O, act, &p->gate[s]);
+        if(rc != NBL_OK) { nbl_rnn_plan_destroy(ctx, p); return rc; }
+    }
+    *out = p;
+    return NBL_OK;
+}
+
+int nbl_rnn_plan_destroy(nbl_ctx *ctx, nbl_rnn_plan *p) {
+    if(!ctx || !p) return NBL_EINVAL;
+    for(int s = 0; s < 3; s++) if(p->gate[s]) nbl_fc_plan_destroy(ctx, p->gate[s]);
+    nbl_free(ctx, p->in_all); nbl_free(ctx, p->states); nbl_free(ctx, p->hid0); nbl_free(ctx, p->tmp);
+    delete p;
+    return NBL_OK;
+}
+
+int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev, unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_rnn_fwd: NULL argument");
+    if(T == 0 || B == 0) return NBL_OK;
+    const size_t rows = (size_t)T * B;
+    if(rows * p->O >= (1ull << 31) || rows * p->I >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_rnn_fwd: tensors of 2^31 elements or more are not supported");
+    int rc;
+    if(p->rows_alloc < rows || p->seqs_alloc < B) {
+        if((rc = nbl_free(ctx, p->in_all)) != NBL_OK || (rc = nbl_free(ctx, p->states)) != NBL_OK ||
+           (rc = nbl_free(ctx, p->hid0)) != NBL_OK || (rc = nbl_free(ctx, p->tmp)) != NBL_OK) return rc;
+        p->in_all = p->states = p->hid0 = p->tmp = NULL; p->rows_alloc = p->seqs_alloc = 0;
+        if((rc = nbl_malloc(ctx, (void**)&p->in_all, rows * p->O * sizeof(float))) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->states, rows * p->O * sizeof(float))) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->hid0, (size_t)B * p->O * sizeof(float))) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->tmp, (size_t)B * p->O * sizeof(float))) != NBL_OK) return rc;
+        p->rows_alloc = rows; p->seqs_alloc = B;
+    }
+    nbl_fc_plan *gi = p->gate[0], *gh = p->gate[1], *go = p->gate[2];
+    // input gate for every step at once: it does not depend on the recurrence
+    if((rc = launch_fc(ctx, x_dev, gi->w_dev, p->in_all, (int)rows, (int)p->O, (int)p->I, gi->g_dev, gi->b_dev,
+                       gi->act, gi->has_scale, &gi->ws_dev, &gi->ws_bytes)) != NBL_OK) return rc;
+    const size_t step = (size_t)B * p->O;
+    const bool one_launch = p->O % 128 == 0 && aligned16(gh->w_dev) && aligned16(p->in_all) && aligned16(p->states) &&
+                            aligned16(p->hid0);
+    for(unsigned t = 0; t < T; t++) {
+        // rnn_layer.cc:103-104: step 0's hidden gate reads the input gate's output, later steps the previous state
+        const float *prev = t == 0 ? p->in_all : p->states + (size_t)(t - 1) * step;
+        const float *in_t = p->in_all + (size_t)t * step;
+        float *state = p->states + (size_t)t * step;
+        if(one_launch) {
+            RnnStepArgs a;
+            a.prev = prev; a.w = gh->w_dev; a.g = gh->g_dev; a.b = gh->b_dev; a.in_t = in_t; a.state = state;
+            a.hid = t == 0 ? p->hid0 : NULL; a.B = (int)B; a.H = (int)p->O; a.act = gh->act;
+            hipLaunchKernelGGL(rnn_step_kernel, dim3(p->O / 32, nbl_div_up(B, 32)), dim3(256), 0, ctx->stream, a);
+            NBL_LAUNCH_CHECK(ctx, "rnn_step_kernel");
+        } else {
+            float *hid = t == 0 ? p->hid0 : p->tmp;
+            if((rc = launch_fc(ctx, prev, gh->w_dev, hid, (int)B, (int)p->O, (int)p->O, gh->g_dev, gh->b_dev,
+                               gh->act, gh->has_scale, &gh->ws_dev, &gh->ws_bytes)) != NBL_OK) return rc;
+            hipLaunchKernelGGL(add_kernel, dim3((unsigned)nbl_div_up_sz(step, 256)), dim3(256), 0, ctx->stream,
+                               in_t, (const float*)hid, state, step);
+            NBL_LAUNCH_CHECK(ctx, "add_kernel");
+        }
+    }
+    // output gate: step 0 reads the hidden gate's output (rnn_layer.cc:116-117), every later step its state;
+    // nothing feeds back, so all later steps are one product
+    if((rc = launch_fc(ctx, p->hid0, go->w_dev, y_dev, (int)B, (int)p->O, (int)p->O, go->g_dev, go->b_dev,
+                       go->act, go->has_scale, &go->ws_dev, &go->ws_bytes)) != NBL_OK) return rc;
+    if(T > 1 && (rc = launch_fc(ctx, p->states + step, go->w_dev, y_dev + step, (int)(rows - B), (int)p->O, (int)p->O,
+                                go->g_dev, go->b_dev, go->act, go->has_scale, &go->ws_dev, &go->ws_bytes)) != NBL_OK) return rc;
+    return NBL_OK;
 }
 
 }  // extern "C"

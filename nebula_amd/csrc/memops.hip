@@ -367,6 +367,29 @@ __global__ __launch_bounds__(1024) void target_prob_sum_kernel(const float *__re
     if(threadIdx.x == 0) *out = red[0];
 }
 
+
+__global__ void clear_u32_kernel(unsigned *p) { *p = 0u; }
+
+// Rows whose label ranks among the k largest entries: one wave per row counts the entries that come
+// before the label in descending order (larger value, or equal value and smaller index); one block per
+// 4 rows; the per-block counts are added with an integer atomic (order-independent).
+__global__ __launch_bounds__(256) void topk_matches_kernel(const float *__restrict__ probs, const unsigned *__restrict__ labels,
+                                                           unsigned rows, unsigned n, unsigned k, unsigned *__restrict__ count) {
+    const unsigned row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if(row >= rows) return;
+    const unsigned l = labels[row];
+    if(l >= n) return;
+    const float *__restrict__ p = probs + (size_t)row * n;
+    const float pl = p[l];
+    unsigned before = 0;
+    for(unsigned j = lane; j < n; j += 64) {
+        const float v = p[j];
+        before += (v > pl || (v == pl && j < l)) ? 1u : 0u;
+    }
+    for(int off = 32; off >= 1; off >>= 1) before += __shfl_down(before, off, 64);
+    if(lane == 0 && before < k) atomicAdd(count, 1u);
+}
+
 }  // namespace
 
 extern "C" {
@@ -553,6 +576,19 @@ int nbl_target_prob_sum(nbl_ctx *ctx, const float *probs_dev, const unsigned *ta
     NBL_REQUIRE(ctx, probs_dev && targets_dev && sum_dev, "nbl_target_prob_sum: NULL pointer");
     hipLaunchKernelGGL(target_prob_sum_kernel, dim3(1), dim3(1024), 0, ctx->stream, probs_dev, targets_dev, rows, n, sum_dev);
     NBL_LAUNCH_CHECK(ctx, "target_prob_sum_kernel");
+    return NBL_OK;
+}
+
+int nbl_topk_matches(nbl_ctx *ctx, const float *probs_dev, const unsigned *labels_dev, unsigned rows, unsigned n,
+                     unsigned k, unsigned *count_dev) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, probs_dev && labels_dev && count_dev, "nbl_topk_matches: NULL pointer");
+    hipLaunchKernelGGL(clear_u32_kernel, dim3(1), dim3(1), 0, ctx->stream, count_dev);     // a kernel, so the call stays capturable
+    NBL_LAUNCH_CHECK(ctx, "clear_u32_kernel");
+    if(rows == 0 || n == 0) return NBL_OK;
+    hipLaunchKernelGGL(topk_matches_kernel, dim3(nbl_div_up(rows, 4)), dim3(256), 0, ctx->stream,
+                       probs_dev, labels_dev, rows, n, k, count_dev);
+    NBL_LAUNCH_CHECK(ctx, "topk_matches_kernel");
     return NBL_OK;
 }
 

@@ -38,6 +38,10 @@ SIGNATURES = {
     "nbl_copy_d2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_sync": (C.c_int, [_vp]),
     "nbl_lstm_fwd_tokens": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
+    "nbl_rnn_pack": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u, _u, C.c_int, C.POINTER(_vp)]),
+    "nbl_rnn_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u]),
+    "nbl_rnn_plan_destroy": (C.c_int, [_vp, _vp]),
+    "nbl_topk_matches": (C.c_int, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "nbl_target_prob_sum": (C.c_int, [_vp, _vp, _vp, _u, _u, _vp]),
     "nbl_image_to_input": (C.c_int, [_vp, _vp, _u, _u, _u, _u, _vp, _u, _u]),
     "nbl_conv2d_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, _u, _u, _u, _u, _u, C.c_int,
@@ -258,6 +262,32 @@ class Ctx:
         self._plans.append(("lstm", p))
         return LstmPlan(self, p, I, H)
 
+    def rnn_pack(self, weight, bias, bn=None, act="linear"):
+        """weight/bias: 3 arrays in file order input, hidden, output gate; bn = (scale3, mean3, var3)."""
+        weight = [_f32(w) for w in weight]
+        bias = [_f32(b) for b in bias]
+        O, I = weight[0].shape
+
+        def arr(xs):
+            return None if xs is None else (_f32p * 3)(*[_fp(a) for a in xs])
+        if bn is not None:
+            bn = [[_f32(a) for a in grp] for grp in bn]
+        sc, mu, var = (None, None, None) if bn is None else bn
+        p = _vp()
+        self.check(lib().nbl_rnn_pack(self.h, arr(weight), arr(bias), arr(sc), arr(mu), arr(var), I, O, ACT[act],
+                                      C.byref(p)))
+        self._plans.append(("rnn", p))
+        return RnnPlan(self, p, I, O)
+
+    def topk_matches(self, probs, labels, k):
+        """rows of probs (DeviceArray [rows][n]) whose label (DeviceArray [rows] uint32) is among the k largest."""
+        rows, n = probs.shape
+        out = self.empty((4,), np.uint32)
+        self.check(lib().nbl_topk_matches(self.h, probs.ptr, labels.ptr, rows, n, k, out.ptr))
+        v = int(out.numpy()[0])
+        out.free()
+        return v
+
     # ---- one-shot ops on DeviceArrays ----
     def im2col(self, x, k, s, p):
         Cc, H, W = x.shape
@@ -345,6 +375,18 @@ class FcPlan:
         assert x.size == B * self.I
         y = out if out is not None else self.ctx.empty((B, self.O))
         self.ctx.check(lib().nbl_fc_fwd(self.ctx.h, self.p, x.ptr, y.ptr, B))
+        return y
+
+
+class RnnPlan:
+    def __init__(self, ctx, p, I, O):
+        self.ctx, self.p, self.I, self.O = ctx, p, I, O
+
+    def __call__(self, x, out=None):
+        T, B, I = x.shape
+        assert I == self.I
+        y = out if out is not None else self.ctx.empty((T, B, self.O))
+        self.ctx.check(lib().nbl_rnn_fwd(self.ctx.h, self.p, x.ptr, y.ptr, T, B))
         return y
 
 

@@ -111,7 +111,9 @@ int nbl_net_layer_flop(nbl_net *n, int i, double *flop) {
         layer_t *l = layer_at(n, i);
         *flop = 0.0;
         if(l->layer_type == CONVOLUTIONAL_LAYER) *flop = static_cast<convolutional_layer_t*>(l)->flop_per_image();
-        else if(l->layer_type == CONNECTED_LAYER) *flop = 2.0 * l->input_size * l->output_size);
+        else if(l->layer_type == CONNECTED_LAYER || l->layer_type == RBM_LAYER) *flop = 2.0 * l->input_size * l->output_size;
+        else if(l->layer_type == RNN_LAYER) *flop = 2.0 * (l->input_size + 2.0 * l->output_size) * l->output_size;
+        else if(l->layer_type == LSTM_LAYER) *flop = 2.0 * (l->input_size + (double)l->output_size) * 4.0 * l->output_size);
 }
 
 int nbl_net_set_input(nbl_net *n, const float *host, size_t count) {
@@ -130,6 +132,12 @@ int nbl_net_accumulate_perplexity(nbl_net *n, const unsigned *label_tokens, size
     NBL_NET_TRY(
         if(!n || !label_tokens || !perplexity) throw std::runtime_error("NULL argument");
         *perplexity = n->net->accumulate_perplexity(label_tokens, count));
+}
+
+int nbl_net_accumulate_topk(nbl_net *n, const unsigned *labels, size_t count, unsigned k, unsigned *matches) {
+    NBL_NET_TRY(
+        if(!n || !labels || !matches) throw std::runtime_error("NULL argument");
+        *matches = n->net->accumulate_topk(labels, count, k));
 }
 
 int nbl_net_forward(nbl_net *n) {

@@ -524,4 +524,97 @@ void lstm_layer_t::_forward_() {
               "nbl_lstm_fwd");
 }
 
+// ---- rnn ------------------------------------------------------------------------------------------
+rnn_layer_t::rnn_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type) :
+    layer_t(m_network, m_prev_layer, m_layer_type), batch_normalize(false),
+    input_gate(NULL), hidden_gate(NULL), output_gate(NULL), plan(NULL) {}
+
+rnn_layer_t::~rnn_layer_t() {
+    if(plan) nbl_rnn_plan_destroy(network->ctx, plan);
+    delete input_gate; delete hidden_gate; delete output_gate;
+}
+
+void rnn_layer_t::init(section_config_t m_section_config) {
+    m_section_config.get_setting("output", &output_size);
+    m_section_config.get_setting("batch_normalize", &batch_normalize);
+    read_activation(m_section_config);
+    if(activation_type == UNDEFINED_ACTIVATION)
+        throw std::runtime_error("Error: undefined activation type undefined_activation");
+    input_size = prev_layer ? prev_layer->output_size : network->input_size;
+    if(!network->time_step || network->batch_size % network->time_step)
+        throw std::runtime_error("Error: batch size is not a multiple of time_steps");
+    // parameter holders: the input gate reads the layer's input, the other two the layer's own width
+    connected_layer_t **slots[3] = { &input_gate, &hidden_gate, &output_gate };
+    layer_t *saved_next = prev_layer ? prev_layer->next_layer : NULL;
+    for(int s = 0; s < 3; s++) {
+        connected_layer_t *sub = new connected_layer_t(network, NULL, CONNECTED_LAYER);
+        sub->allocate_output = false;
+        sub->input_size = s == 0 ? input_size : output_size;
+        sub->init(m_section_config);
+        *slots[s] = sub;
+    }
+    if(prev_layer) prev_layer->next_layer = saved_next;
+    alloc_output();
+}
+
+void rnn_layer_t::init_weight(std::fstream &m_weight_file) {
+    input_gate->init_weight(m_weight_file);
+    hidden_gate->init_weight(m_weight_file);
+    output_gate->init_weight(m_weight_file);
+    pack();
+}
+
+void rnn_layer_t::init_weight() {
+    input_gate->init_weight(); hidden_gate->init_weight(); output_gate->init_weight();
+    pack();
+}
+
+void rnn_layer_t::store_weight(std::fstream &m_weight_file) {
+    input_gate->store_weight(m_weight_file);
+    hidden_gate->store_weight(m_weight_file);
+    output_gate->store_weight(m_weight_file);
+}
+
+void rnn_layer_t::weight_fields(std::vector<weight_field_t> &out) const {
+    input_gate->weight_fields(out); hidden_gate->weight_fields(out); output_gate->weight_fields(out);
+}
+
+void rnn_layer_t::pack() {
+    if(!network->ctx) return;          // dry-run network
+    if(plan) { nbl_rnn_plan_destroy(network->ctx, plan); plan = NULL; }
+    connected_layer_t *order[3] = { input_gate, hidden_gate, output_gate };
+    const float *w[3], *b[3], *sc[3], *mu[3], *var[3];
+    for(int s = 0; s < 3; s++) {
+        w[s] = order[s]->weight.data(); b[s] = order[s]->bias.data();
+        sc[s] = batch_normalize ? order[s]->scale.data() : NULL;
+        mu[s] = batch_normalize ? order[s]->rolling_mean.data() : NULL;
+        var[s] = batch_normalize ? order[s]->rolling_variance.data() : NULL;
+    }
+    nbl_check(network->ctx,
+              nbl_rnn_pack(network->ctx, w, b, batch_normalize ? sc : NULL, batch_normalize ? mu : NULL,
+                           batch_normalize ? var : NULL, input_size, output_size, (int)activation_type, &plan),
+              "nbl_rnn_pack");
+}
+
+void rnn_layer_t::_forward_() {
+    if(!plan) throw std::runtime_error("Error: rnn layer has no weights (init_weight not called)");
+    nbl_check(network->ctx,
+              nbl_rnn_fwd(network->ctx, plan, input_dev(), output_data_dev, network->time_step,
+                          network->batch_size / network->time_step),
+              "nbl_rnn_fwd");
+}
+
+// ---- rbm ------------------------------------------------------------------------------------------
+rbm_layer_t::rbm_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type) :
+    connected_layer_t(m_network, m_prev_layer, m_layer_type) {}
+
+// rbm_layer.cc:69-90 reads output, k_step and activation; there is no batch_normalize key for it to honour
+void rbm_layer_t::init(section_config_t m_section_config) {
+    connected_layer_t::init(m_section_config);
+    if(batch_normalize) {
+        batch_normalize = false;
+        scale.clear(); rolling_mean.clear(); rolling_variance.clear();
+    }
+}
+
 }  // namespace nebula

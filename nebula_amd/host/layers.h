@@ -199,5 +199,32 @@ private:
     nbl_lstm_plan *plan;
 };
 
+// models/layers/rnn_layer.h: three connected sub-layers (input, hidden, output gate) sharing the section's
+// output size, activation and batch_normalize
+class rnn_layer_t : public layer_t {
+public:
+    rnn_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type);
+    ~rnn_layer_t();
+    void init(section_config_t m_section_config);
+    void init_weight(std::fstream &m_weight_file);
+    void init_weight();
+    void store_weight(std::fstream &m_weight_file);
+    void _forward_();
+    void weight_fields(std::vector<weight_field_t> &out) const;
+private:
+    void pack();
+    bool batch_normalize;
+    connected_layer_t *input_gate, *hidden_gate, *output_gate;    // file order
+    nbl_rnn_plan *plan;
+};
+
+// models/layers/rbm_layer.h at inference: forward() is a connected layer without batchnorm
+// (rbm_layer.cc:345-374); the file holds hidden_bias[O] then weight[O][I] (:150-153).
+class rbm_layer_t : public connected_layer_t {
+public:
+    rbm_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type);
+    void init(section_config_t m_section_config);
+};
+
 }  // namespace nebula
 #endif

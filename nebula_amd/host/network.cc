@@ -67,7 +67,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
     last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false),
-    cumulative_cost(0.0f), rows_seen(0), image_staging_dev(NULL), image_staging_bytes(0), tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL) {
+    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), image_staging_dev(NULL), image_staging_bytes(0), tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
@@ -146,6 +146,8 @@ void inference_net_t::build(config_t &config) {
         else if(sc.name == "softmax")  { layer = new softmax_layer_t(this, prev, SOFTMAX_LAYER); output_layer = layer; }
         else if(sc.name == "cost")       layer = new cost_layer_t(this, prev, COST_LAYER);
         else if(sc.name == "lstm")       layer = new lstm_layer_t(this, prev, LSTM_LAYER);
+        else if(sc.name == "rnn")        layer = new rnn_layer_t(this, prev, RNN_LAYER);
+        else if(sc.name == "rbm")        layer = new rbm_layer_t(this, prev, RBM_LAYER);
         else throw std::runtime_error("Error: unknown layer type " + sc.name);
         if(layers.empty()) input_layer = layer;
         layers.push_back(layer);            // owned from here on, also if init() throws
@@ -158,7 +160,7 @@ void inference_net_t::build(config_t &config) {
             if(layers[i]->layer_type == SHORTCUT_LAYER && layers[i - 1]->layer_type == CONVOLUTIONAL_LAYER)
                 static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
     for(unsigned i = 0; i < num_layers; i++)
-        if(layers[i]->layer_type == LSTM_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
+        if(layers[i]->layer_type == LSTM_LAYER || layers[i]->layer_type == RNN_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
 }
 
 void inference_net_t::init_data(const std::string) {
@@ -223,6 +225,22 @@ void inference_net_t::set_input_images(const unsigned char *host, unsigned image
     nbl_check(ctx, nbl_h2d(ctx, image_staging_dev, host, bytes), "nbl_h2d(images)");
     nbl_check(ctx, nbl_image_to_input(ctx, image_staging_dev, images, height, width, input_channel, input_data_dev,
                                       input_height, input_width), "nbl_image_to_input");
+}
+
+unsigned inference_net_t::accumulate_topk(const unsigned *labels_host, size_t count, unsigned k) {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
+    if(!output_layer) throw std::runtime_error("Error: network has no layers");
+    const size_t rows = last_step_only && is_recurrent ? batch_size / time_step : batch_size;
+    if(count != rows) throw std::runtime_error("Error: labels have the wrong size");
+    if(!labels_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&labels_dev, (size_t)batch_size * sizeof(unsigned)), "nbl_malloc(labels)");
+    if(!cost_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&cost_dev, 16), "nbl_malloc(cost)");
+    nbl_check(ctx, nbl_h2d(ctx, labels_dev, labels_host, count * sizeof(unsigned)), "nbl_h2d(labels)");
+    nbl_check(ctx, nbl_topk_matches(ctx, output_layer->output_data_dev, labels_dev, (unsigned)rows, output_layer->output_size, k,
+                                    reinterpret_cast<unsigned*>(cost_dev)), "nbl_topk_matches");
+    unsigned found = 0;
+    nbl_check(ctx, nbl_d2h(ctx, &found, cost_dev, sizeof(unsigned)), "nbl_d2h(matches)");
+    topk_matches += found;
+    return topk_matches;
 }
 
 void inference_net_t::load_data(const unsigned) {}

@@ -91,6 +91,10 @@ public:
     // the output layer to cumulative_cost and returns exp(-log2(cumulative_cost / rows seen so far)).
     float accumulate_perplexity(const unsigned *label_tokens_host, size_t count);
     float cumulative_cost; size_t rows_seen;
+    // convolutional_t::print_results(), test branch (convolutional.cc:428-447): running count of rows whose label
+    // is among the output layer's k largest entries.
+    unsigned accumulate_topk(const unsigned *labels_host, size_t count, unsigned k);
+    unsigned topk_matches;
     void run(const std::string m_output_weight = "");
     bool recurrent() const { return is_recurrent; }
 

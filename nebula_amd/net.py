@@ -29,6 +29,7 @@ SIGNATURES = {
     "nbl_net_set_input_images": (C.c_int, [_vp, _vp, _u, _u, _u]),
     "nbl_net_set_input_tokens": (C.c_int, [_vp, _vp, C.c_size_t]),
     "nbl_net_accumulate_perplexity": (C.c_int, [_vp, _vp, C.c_size_t, C.POINTER(C.c_float)]),
+    "nbl_net_accumulate_topk": (C.c_int, [_vp, _vp, C.c_size_t, _u, C.POINTER(_u)]),
     "nbl_net_forward": (C.c_int, [_vp]),
     "nbl_net_sync": (C.c_int, [_vp]),
     "nbl_net_forward_timed": (C.c_int, [_vp, C.POINTER(C.c_float)]),
@@ -145,6 +146,12 @@ class Network:
         t = np.ascontiguousarray(label_tokens, np.uint32)
         out = C.c_float()
         self._check(lib().nbl_net_accumulate_perplexity(self.h, t.ctypes.data, t.size, C.byref(out)))
+        return out.value
+
+    def accumulate_topk(self, labels, k):
+        t = np.ascontiguousarray(labels, np.uint32)
+        out = _u()
+        self._check(lib().nbl_net_accumulate_topk(self.h, t.ctypes.data, t.size, k, C.byref(out)))
         return out.value
 
     def forward(self):

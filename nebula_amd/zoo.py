@@ -82,6 +82,36 @@ def lstm_cfg(batch=64, time_steps=64, input_size=1024, hidden=1024, layers=2, cl
     return s
 
 
+def rnn_cfg(batch=32, time_steps=40, input_size=8713, hidden=1024, layers=5, last_step_only=False):
+    """benchmarks/rnn_large/network.cfg: five normalised [rnn] layers of 1024, projection back to the vocabulary."""
+    s = "[net]\nbatch=%d\ninput_size=%d\ntime_steps=%d\n" % (batch, input_size, time_steps)
+    if last_step_only:
+        s += "last_step_only=1\n"
+    for _ in range(layers):
+        s += "\n[rnn]\nbatch_normalize=1\noutput=%d\nactivation=linear\n" % hidden
+    s += _fc(input_size, "linear") + _TAIL
+    return s
+
+
+def dbn_cfg(batch=32):
+    """benchmarks/dbn_large/network.cfg: four [rbm] layers (2000, 1000, 500, 30, logistic) on 3x128x128 inputs."""
+    s = _net(batch, 128, 128, 3)
+    for out in (2000, 1000, 500, 30):
+        s += "\n[rbm]\noutput=%d\nk_step=1\nactivation=logistic\n" % out
+    s += _fc(62, "linear") + _TAIL
+    return s
+
+
+def mlp_cfg(batch=32):
+    """benchmarks/mlp_large/network.cfg: 2500-2000-1500-1000-500 relu, 62 classes, 3x128x128 inputs."""
+    s = _net(batch, 128, 128, 3)
+    for out in (2500, 2000, 1500, 1000, 500):
+        s += _fc(out, "relu")
+    s += _fc(62, "linear") + _TAIL
+    return s
+
+
 WORKLOADS = {
     "conv1": conv1_pool_cfg, "alexnet": alexnet_cfg, "vgg16": vgg16_cfg, "resnet50": resnet50_cfg, "lstm": lstm_cfg,
+    "rnn": rnn_cfg, "dbn": dbn_cfg, "mlp": mlp_cfg,
 }

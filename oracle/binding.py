@@ -96,6 +96,9 @@ def oracle():
         lib.orc_image_to_input.argtypes = [C.c_void_p, _u, _u, _u, _f32p, _u, _u]
         lib.orc_resize_linear_u8.argtypes = [C.c_void_p, _u, _u, _u, C.c_void_p, _u, _u]
         pp = C.POINTER(_f32p)
+        lib.orc_rnn_forward.argtypes = [_f32p, pp, pp, pp, pp, pp, _f32p, _u, _u, _u, _u, _u]
+        lib.orc_topk_matches.argtypes = [_f32p, C.c_void_p, _u, _u, _u]
+        lib.orc_topk_matches.restype = _u
         lib.orc_lstm_forward.argtypes = [_f32p, pp, pp, pp, pp, pp, _f32p, _f32p, _u, _u, _u, _u, _u]
         _oracle = lib
     return _oracle
@@ -282,6 +285,28 @@ def lstm_forward(x, weight, bias, bn=None, act="linear", want_cell=False):
     return (y, cell) if want_cell else y
 
 
+def rnn_forward(x, weight, bias, bn=None, act="linear"):
+    """x [T,B,I]; weight/bias: 3 arrays in file order input, hidden, output gate; bn = (scale3, mean3, var3)."""
+    x = _f32(x)
+    T, B, I = x.shape
+    weight = [_f32(w) for w in weight]
+    bias = [_f32(b) for b in bias]
+    O = weight[0].shape[0]
+    y = np.empty((T, B, O), np.float32)
+    if bn is not None:
+        bn = [[_f32(a) for a in grp] for grp in bn]
+    sc, mu, var = (None, None, None) if bn is None else bn
+    oracle().orc_rnn_forward(_fp(x), _ptr_array(weight), _ptr_array(bias), _ptr_array(sc), _ptr_array(mu),
+                             _ptr_array(var), _fp(y), T, B, I, O, ACT[act])
+    return y
+
+
+def topk_matches(probs, labels, k):
+    probs = _f32(probs); labels = np.ascontiguousarray(labels, np.uint32)
+    rows, n = probs.shape
+    return int(oracle().orc_topk_matches(_fp(probs), labels.ctypes.data, rows, n, k))
+
+
 # ------------------------------------------------------------------------------------------------
 # network.cfg handling (common/config.cc:44-75: spaces stripped, '#' comments, keys AND values
 # lower-cased, unknown keys ignored)
@@ -385,6 +410,14 @@ def plan_network(cfg_text, batch=None):
             O = g("output", 0)
             specs.append(LayerSpec(name, I=size, H=O, bn=bn, act=act, out=(1, 1, 1)))
             cur = (1, 1, 1, O)
+        elif name == "rnn":
+            O = g("output", 0)
+            specs.append(LayerSpec(name, I=size, O=O, bn=bn, act=act, out=(1, 1, 1)))
+            cur = (1, 1, 1, O)
+        elif name == "rbm":     # rbm_layer.cc:70-90, forward = connected without batchnorm (:345-374)
+            O = g("output", 0)
+            specs.append(LayerSpec(name, I=size, O=O, bn=False, act=act, out=(1, 1, 1)))
+            cur = (1, 1, 1, O)
         else:
             raise ValueError("unknown layer type " + name)
         specs[-1].out_size = cur[3] if name not in ("shortcut", "softmax", "cost") else size
@@ -404,6 +437,13 @@ def weight_layout(specs):
             fields += [(li, "bias", (sp.O,)), (li, "weight", (sp.O, sp.I))]
             if sp.bn:
                 fields += [(li, "scale", (sp.O,)), (li, "mean", (sp.O,)), (li, "var", (sp.O,))]
+        elif sp.kind == "rbm":          # rbm_layer.cc:150-153: hidden_bias, weight
+            fields += [(li, "bias", (sp.O,)), (li, "weight", (sp.O, sp.I))]
+        elif sp.kind == "rnn":          # rnn_layer.cc:73-77: input, hidden, output gate, each a connected layer's fields
+            for sub, fan_in in (("in", sp.I), ("hid", sp.O), ("out", sp.O)):
+                fields += [(li, sub + ".bias", (sp.O,)), (li, sub + ".weight", (sp.O, fan_in))]
+                if sp.bn:
+                    fields += [(li, sub + ".scale", (sp.O,)), (li, sub + ".mean", (sp.O,)), (li, sub + ".var", (sp.O,))]
         elif sp.kind == "lstm":
             for sub in ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU"):
                 fan_in = sp.H if sub[1] == "W" else sp.I
@@ -462,6 +502,16 @@ class OracleNet:
                 cur = softmax_forward(cur.reshape(-1, sp.n))
             elif sp.kind in ("dropout", "cost"):
                 pass
+            elif sp.kind == "rbm":
+                rows = cur.shape[0] * (cur.shape[1] if self.net["recurrent"] and cur.ndim == 3 else 1)
+                cur = connected_forward(cur.reshape(rows, -1), wt["weight"], wt["bias"], None, sp.act)
+            elif sp.kind == "rnn":
+                subs = ("in", "hid", "out")
+                bn = None
+                if sp.bn:
+                    bn = ([wt[q + ".scale"] for q in subs], [wt[q + ".mean"] for q in subs], [wt[q + ".var"] for q in subs])
+                cur = rnn_forward(cur.reshape(T, -1, sp.I), [wt[q + ".weight"] for q in subs],
+                                  [wt[q + ".bias"] for q in subs], bn, sp.act)
             elif sp.kind == "lstm":
                 subs = ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU")
                 bn = None

@@ -476,6 +476,53 @@ float orc_perplexity(float cumulative_cost, unsigned rows_seen) {
 }
 
 /* ---------------------------------------------------------------------------------------
+ * RNN layer, rnn_layer.cc:91-141.  Three connected sub-layers in file order input, hidden,
+ * output (rnn_layer.cc:73-77), all initialised from the same section (same output size,
+ * activation and batch_normalize).  Per time step, on the B rows of that step:
+ *   in_t  = input_gate(x_t)
+ *   hid_t = hidden_gate(t == 0 ? in_0 : state_{t-1})     (:103-104: without an argument the
+ *           sub-layer reads its prev_layer, which is the input gate)
+ *   state = 0; state += in_t; state += hid_t              (:108-115, two axpy with alpha 1)
+ *   out_t = output_gate(t == 0 ? hid_0 : state)           (:116-117: prev_layer is the hidden gate)
+ * The layer's output is the output gate's [T][B][O].  Every sub-layer call is a full
+ * connected forward (GEMM nt, [BN], bias, activation).
+ * ------------------------------------------------------------------------------------- */
+void orc_rnn_forward(const float *x, const float *const *weight, const float *const *bias,
+                     const float *const *scale, const float *const *mean, const float *const *var,
+                     float *y, unsigned T, unsigned B, unsigned I, unsigned O, unsigned act) {
+    const size_t n = (size_t)B * O;
+    float *in = (float*)malloc(sizeof(float) * n), *hid = (float*)malloc(sizeof(float) * n);
+    float *state = (float*)calloc(n, sizeof(float));
+    for(unsigned t = 0; t < T; t++) {
+        orc_connected_forward(x + (size_t)t * B * I, weight[0], bias[0], scale ? scale[0] : NULL,
+                              mean ? mean[0] : NULL, var ? var[0] : NULL, in, B, I, O, act);
+        orc_connected_forward(t ? state : in, weight[1], bias[1], scale ? scale[1] : NULL,
+                              mean ? mean[1] : NULL, var ? var[1] : NULL, hid, B, O, O, act);
+        for(size_t e = 0; e < n; e++) { float s = 0.0f; s += 1.0f * in[e]; s += 1.0f * hid[e]; state[e] = s; }
+        orc_connected_forward(t ? state : hid, weight[2], bias[2], scale ? scale[2] : NULL,
+                              mean ? mean[2] : NULL, var ? var[2] : NULL, y + (size_t)t * n, B, O, O, act);
+    }
+    free(in); free(hid); free(state);
+}
+
+/* convolutional_t::print_results(), test branch (models/networks/convolutional.cc:428-447): per row the
+ * class indices are sorted by descending output and the label counts as a match when it is among the first
+ * top_k.  The reference sorts with std::sort, whose order among equal outputs is unspecified; here equal
+ * outputs keep ascending index order (a stable sort), which is what decides a tie at the k-th place. */
+unsigned orc_topk_matches(const float *probs, const unsigned *labels, unsigned rows, unsigned n, unsigned k) {
+    unsigned matches = 0;
+    for(unsigned r = 0; r < rows; r++) {
+        const float *p = probs + (size_t)r * n;
+        const unsigned l = labels[r];
+        if(l >= n) continue;
+        unsigned before = 0;
+        for(unsigned j = 0; j < n; j++) if(p[j] > p[l] || (p[j] == p[l] && j < l)) before++;
+        if(before < k) matches++;
+    }
+    return matches;
+}
+
+/* ---------------------------------------------------------------------------------------
  * LSTM, lstm_layer.cc:233-346.  Sub-layer slots in file order (lstm_layer.cc:194-206):
  *   0 iW  1 fW  2 oW  3 cW  4 iU  5 fU  6 oU  7 cU
  * Per step: every sub-layer runs a full connected forward (GEMM nt, [BN], bias, the section's

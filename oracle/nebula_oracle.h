@@ -93,6 +93,17 @@ void orc_shortcut_forward(const float *prev, const float *conn, float *out, unsi
 /* models/layers/softmax_layer.cc:85-106 */
 void orc_softmax_forward(const float *x, float *y, unsigned rows, unsigned n);
 
+/* rnn_layer_t::forward (models/layers/rnn_layer.cc:91-141).  weight/bias (and scale/mean/var or three
+ * NULLs): 3 arrays in file order input gate [O][I], hidden gate [O][O], output gate [O][O].
+ * x [T][B][I] -> y [T][B][O]. */
+void orc_rnn_forward(const float *x, const float *const *weight, const float *const *bias,
+                     const float *const *scale, const float *const *mean, const float *const *var,
+                     float *y, unsigned T, unsigned B, unsigned I, unsigned O, unsigned act);
+
+/* Top-k matches as convolutional_t::print_results() counts them (models/networks/convolutional.cc:428-447);
+ * ties keep ascending class order (the reference's std::sort leaves them unspecified). */
+unsigned orc_topk_matches(const float *probs, const unsigned *labels, unsigned rows, unsigned n, unsigned k);
+
 /* recurrent_t::print_results() (models/networks/recurrent.cc:239-247): sum of label * output with one-hot
  * labels, and the "perplexity" figure the driver prints from it. */
 float orc_target_prob_sum(const float *probs, const unsigned *targets, unsigned rows, unsigned n);

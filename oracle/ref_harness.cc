@@ -36,6 +36,8 @@
 #include "softmax_layer.h"
 #include "cost_layer.h"
 #include "lstm_layer.h"
+#include "rnn_layer.h"
+#include "rbm_layer.h"
 // The maxpool argmax table is a private member of the reference class; the
 // harness has to read it, so access control (only) is lifted for this header.
 #define private public
@@ -83,6 +85,8 @@ struct probe_net_t : public network_t {
             else if(sc.name == "softmax") { layer = new softmax_layer_t(this, prev, SOFTMAX_LAYER); output_layer = layer; }
             else if(sc.name == "cost") layer = new cost_layer_t(this, prev, COST_LAYER);
             else if(sc.name == "lstm") layer = new lstm_layer_t(this, prev, LSTM_LAYER);
+            else if(sc.name == "rnn") layer = new rnn_layer_t(this, prev, RNN_LAYER);
+            else if(sc.name == "rbm") layer = new rbm_layer_t(this, prev, RBM_LAYER);
             else { fprintf(stderr, "ref_harness: unknown section %s\n", sc.name.c_str()); exit(1); }
             if(!layers.size()) input_layer = layer;
             layer->init(sc);

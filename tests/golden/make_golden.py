@@ -226,6 +226,77 @@ activation=linear
 groups=1
 """, "normal")
 
+# rnn_layer.cc: three connected sub-layers per [rnn]; step 0 takes its hidden and output gates' inputs from
+# the neighbouring sub-layer instead of the running state.
+CASES["rnn_plain"] = ("""
+[net]
+batch=3
+input_size=7
+time_steps=4
+
+[rnn]
+output=6
+activation=relu
+
+[rnn]
+output=5
+activation=linear
+
+[connected]
+output=8
+activation=linear
+
+[softmax]
+""", "normal")
+
+# The shipped rnn cfgs (benchmarks/rnn_large/network.cfg) normalize every sub-layer.
+CASES["rnn_bn_leaky"] = ("""
+[net]
+batch=2
+input_size=9
+time_steps=5
+
+[rnn]
+batch_normalize=1
+output=7
+activation=leaky
+
+[connected]
+output=6
+activation=linear
+
+[softmax]
+""", "normal")
+
+# benchmarks/dbn_*/network.cfg: [rbm] layers run as connected layers without batchnorm at inference.
+CASES["dbn_small"] = ("""
+[net]
+batch=4
+height=6
+width=5
+channels=3
+
+[rbm]
+output=20
+k_step=1
+activation=logistic
+
+[rbm]
+output=9
+k_step=1
+activation=logistic
+
+[connected]
+output=5
+activation=linear
+
+[softmax]
+""", "uniform")
+
+# Seeds of the fixtures already committed stay what they were; new cases get their own.
+SEEDS = {"alexnet_conv1_small": 1000, "convnet_mixed": 1001, "lstm_bn_tanh": 1002, "lstm_plain": 1003,
+         "resnet_shortcuts": 1004, "rnn_plain": 2007, "rnn_bn_leaky": 2006, "dbn_small": 2005}
+
 
 def make_weights(specs, rng):
     parts = []
@@ -249,8 +320,11 @@ def make_weights(specs, rng):
 def main():
     if ob.ref() is None:
         sys.exit("the reference tree is not present: golden vectors can only be written in the authoring container")
-    for seed, (name, (cfg, dist)) in enumerate(sorted(CASES.items())):
-        rng = np.random.default_rng(1000 + seed)
+    only = set(sys.argv[1:])       # optional: names of the cases to (re)write
+    for name, (cfg, dist) in sorted(CASES.items()):
+        if only and name not in only:
+            continue
+        rng = np.random.default_rng(SEEDS[name])
         net, specs = ob.plan_network(cfg)
         rn = ob.RefNet(cfg)
         n_in = rn.input_size * rn.batch_size
@@ -272,6 +346,8 @@ def main():
         np.savez_compressed(path, **data)
         print("%-22s layers=%2d  %6.1f KB" % (name, len(outs), os.path.getsize(path) / 1024))
 
+    if only and "activations" not in only:
+        return
     # all 13 activations on a fixed vector with the awkward points in it
     rng = np.random.default_rng(77)
     x = (rng.standard_normal(4096) * 3).astype(np.float32)

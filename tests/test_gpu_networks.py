@@ -311,3 +311,20 @@ def test_recurrent_driver_contract_tokens_and_perplexity():
         net.set_input(x)                          # back to the dense input
         net.forward()
         np.testing.assert_array_equal(net.output(0).view(np.uint32), dense[0].view(np.uint32))
+
+
+def test_image_driver_topk_count(golden_dir):
+    """Running top-k match count of the image driver on the DBN fixture's probabilities."""
+    from nebula_amd.net import Network
+    print("CASE topk through network", flush=True)
+    g = np.load(os.path.join(golden_dir, "dbn_small.npz"))
+    with Network(str(g["cfg"])) as net:
+        net.load_weight_blob(g["weights"])
+        net.set_input(g["input"])
+        net.forward()
+        probs = g["out_03"].reshape(net.batch_size, -1)
+        labels = np.array([0, 3, 1, 4], np.uint32)
+        total = 0
+        for k in (1, 2):
+            total += ob.topk_matches(probs, labels, k)
+            assert net.accumulate_topk(labels, k) == total

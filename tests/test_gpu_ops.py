@@ -408,6 +408,48 @@ def test_target_prob_sum_and_perplexity(ctx):
         assert abs(got - float(p[np.arange(rows), t].astype(np.float64).sum())) <= 1e-5 * abs(want)
 
 
+RNN = [(3, 2, 5, 4, False, "linear"), (4, 3, 9, 7, True, "leaky"), (5, 37, 48, 128, False, "relu"),
+       (4, 64, 96, 256, True, "linear"), (1, 5, 16, 128, False, "tanh"), (3, 32, 200, 384, True, "relu")]
+
+
+@pytest.mark.parametrize("case", RNN)
+def test_rnn_matches_oracle(ctx, case):
+    """rnn_layer_t::forward, incl. its step-0 wiring; widths that are multiples of 128 take the fused step kernel."""
+    announce("rnn", case)
+    T, B, I, O, bn, act = case
+    rng = np.random.default_rng(T * 1000 + B + I + O)
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    fan = (I, O, O)
+    wt = [(rng.standard_normal((O, f)) * np.sqrt(1.0 / f)).astype(np.float32) for f in fan]
+    bs = [(rng.standard_normal(O) * 0.1).astype(np.float32) for _ in fan]
+    bnp = None
+    if bn:
+        bnp = ([rng.uniform(0.8, 1.2, O).astype(np.float32) for _ in fan],
+               [(rng.standard_normal(O) * 0.1).astype(np.float32) for _ in fan],
+               [rng.uniform(0.5, 1.5, O).astype(np.float32) for _ in fan])
+    want = ob.rnn_forward(x, wt, bs, bnp, act)
+    plan = ctx.rnn_pack(wt, bs, bnp, act)
+    got = plan(ctx.array(x)).numpy()
+    assert rel(got, want) <= TOL, rel(got, want)
+    for t in range(T):                      # every step on its own scale (step 0 is wired differently)
+        assert rel(got[t], want[t]) <= TOL, (t, rel(got[t], want[t]))
+    np.testing.assert_array_equal(bits(plan(ctx.array(x)).numpy()), bits(got))
+
+
+def test_topk_matches(ctx):
+    announce("topk")
+    rng = np.random.default_rng(41)
+    for rows, n, k in ((1, 5, 1), (37, 11, 3), (128, 1000, 5), (9, 70, 70)):
+        p = rng.random((rows, n), dtype=np.float32)
+        p[::3, : n // 2] = p[::3, n // 2: 2 * (n // 2)]          # ties, also at the k-th place
+        labels = rng.integers(0, n, rows).astype(np.uint32)
+        want = ob.topk_matches(p, labels, k)
+        got = ctx.topk_matches(ctx.array(p), ctx.array(labels, dtype=np.uint32), k)
+        assert got == want, (rows, n, k, got, want)
+        order = np.argsort(-p.astype(np.float64), axis=1, kind="stable")
+        assert want == int(sum(labels[r] in order[r, :k] for r in range(rows)))
+
+
 def test_error_paths(ctx):
     from nebula_amd import hip
     import ctypes as C

@@ -19,7 +19,8 @@ def bits(a):
 
 
 def test_fixtures_present():
-    assert {"alexnet_conv1_small", "convnet_mixed", "resnet_shortcuts", "lstm_plain", "lstm_bn_tanh"} <= set(NETS)
+    assert {"alexnet_conv1_small", "convnet_mixed", "resnet_shortcuts", "lstm_plain", "lstm_bn_tanh",
+            "rnn_plain", "rnn_bn_leaky", "dbn_small"} <= set(NETS)
 
 
 @pytest.mark.parametrize("name", NETS)
