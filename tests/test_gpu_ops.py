@@ -287,7 +287,10 @@ def test_shortcut_bit_exact(ctx, dims, act):
 
 FC = [(7, 60, 11, False, "linear"), (32, 512, 1000, False, "relu"), (64, 2048, 1000, False, "linear"),
       (128, 1024, 256, True, "leaky"), (5, 33, 3, True, "logistic"), (33, 4096, 130, False, "relu"),
-      (1, 256, 64, False, "tanh")]
+      (1, 256, 64, False, "tanh"),
+      # small batches stream the weight matrix: ragged k tails, neuron tails, one and two batch tiles, split and unsplit
+      (32, 2500, 2000, False, "relu"), (64, 25088, 96, True, "relu"), (17, 1500, 1000, False, "logistic"),
+      (48, 500, 62, True, "linear"), (64, 260, 33, False, "relu"), (2, 49152, 40, False, "relu")]
 
 
 @pytest.mark.parametrize("case", FC)
