@@ -213,6 +213,133 @@ void gemm_nt_kernel(const GemmArgs a) {
     }
 }
 
+// Small-batch fully connected product (M <= 64 rows): the layer is a stream of the [N][K] weight matrix
+// from HBM, so what matters is how many bytes each CU keeps in flight.  Same tiling and LDS layout as
+// gemm_nt_kernel with a 32*MT x 128 block tile, but the global loads run through a ring of four register
+// stages: while k-tile t is multiplied, tiles t+2, t+3 and t+4 are on their way (a single stage covers
+// about a quarter of the HBM latency and held the stream to 3.2 TB/s).  Every load is issued
+// unconditionally (past the end the last tile is re-read and ignored) so that the compiler waits per
+// stage, not for everything.  Output: raw partial sums part[blockIdx.z][M][N] or, with one k chunk,
+// act(sum * g + b).
+template<int MT, int EPI>
+__global__ __launch_bounds__(256)
+void fc_stream_kernel(const GemmArgs a) {
+    constexpr int BK = GEMM_BK, LD = GEMM_LD, NTHREADS = 256, DEPTH = 4;
+    constexpr int BM = MT * 32, BN = 128;
+    constexpr int RA = BM * 8 / NTHREADS, RB = BN * 8 / NTHREADS;
+    __shared__ __attribute__((aligned(16))) float As[2][BM][LD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN][LD];
+    const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int n0 = blockIdx.x * BN;
+    const int k_begin = blockIdx.z * a.k_chunk;
+    const int k_end = min(a.K, k_begin + a.k_chunk);
+    const int nkt = (k_end - k_begin + BK - 1) / BK;
+    if(nkt <= 0) return;
+
+    struct Stage { float4 a[RA], b[RB]; bool valid; };
+    Stage st0, st1, st2, st3;           // named, not an array: an indexed array of stages ends up in scratch memory
+    static_assert(DEPTH == 4, "the ring below is written out for four stages");
+    // Unconditional 16-byte loads (rows 16-byte aligned, K % 4 == 0): a row past the matrix repeats the last
+    // row (its products are never stored), a k past the chunk re-reads the chunk's last four values and is
+    // replaced by zeros; no branch, so nothing makes the compiler wait for more than the stage it needs.
+    const int acol = (tid & 7) * 4;
+    const float *__restrict__ arow[RA];
+    const float *__restrict__ brow[RB];
+    #pragma unroll
+    for(int r = 0; r < RA; r++) arow[r] = a.A + (size_t)min((tid + r * NTHREADS) >> 3, a.M - 1) * a.lda;
+    #pragma unroll
+    for(int r = 0; r < RB; r++) brow[r] = a.Bw + (size_t)min(n0 + ((tid + r * NTHREADS) >> 3), a.N - 1) * a.ldb;
+    auto load_tile = [&](Stage &s, int kt) {
+        const int k = k_begin + min(kt, nkt - 1) * BK + acol;
+        const bool valid = k < k_end;
+        const int kk = valid ? k : k_end - 4;
+        s.valid = valid;            // the zeroing happens when the stage is written to LDS: touching the values
+                                    // here would make the loads wait for themselves
+        #pragma unroll
+        for(int r = 0; r < RA; r++) s.a[r] = *reinterpret_cast<const float4*>(arow[r] + kk);
+        #pragma unroll
+        for(int r = 0; r < RB; r++) s.b[r] = *reinterpret_cast<const float4*>(brow[r] + kk);
+    };
+    // (component-wise selects: a select between two whole float4 objects is compiled through scratch memory)
+    auto store_tile = [&](const Stage &s, int buf) {
+        #pragma unroll
+        for(int r = 0; r < RA; r++) {
+            const int v = tid + r * NTHREADS;
+            const float4 t = s.a[r];
+            *reinterpret_cast<float4*>(&As[buf][v >> 3][(v & 7) * 4]) =
+                make_float4(s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f);
+        }
+        #pragma unroll
+        for(int r = 0; r < RB; r++) {
+            const int v = tid + r * NTHREADS;
+            const float4 t = s.b[r];
+            *reinterpret_cast<float4*>(&Bs[buf][v >> 3][(v & 7) * 4]) =
+                make_float4(s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f);
+        }
+    };
+    floatx16 acc[MT];
+    #pragma unroll
+    for(int i = 0; i < MT; i++)
+        #pragma unroll
+        for(int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+    auto compute_tile = [&](int buf) {
+        #pragma unroll
+        for(int q = 0; q < 4; q++) {
+            const float4 bv = *reinterpret_cast<const float4*>(&Bs[buf][wn * 32 + l32][half * 16 + q * 4]);
+            #pragma unroll
+            for(int i = 0; i < MT; i++) {
+                const float4 av = *reinterpret_cast<const float4*>(&As[buf][i * 32 + l32][half * 16 + q * 4]);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc[i], 0, 0, 0);
+            }
+        }
+    };
+
+    load_tile(st0, 0); load_tile(st1, 1); load_tile(st2, 2); load_tile(st3, 3);
+    store_tile(st0, 0);
+    __syncthreads();
+    // k-tile t travels through stage t % 4 into LDS buffer t % 2.  One step: refill the stage that was written
+    // to LDS one step ago with tile t+4, multiply tile t, write tile t+1 (past the end: a repeat of the last
+    // tile, never multiplied) into the other buffer.
+    #define NBL_FC_STEP(U, CUR, NEXT)                                   \
+        if(kt + U < nkt) {                                              \
+            load_tile(CUR, kt + U + DEPTH);                             \
+            compute_tile(U & 1);                                        \
+            store_tile(NEXT, (U + 1) & 1);                              \
+            __syncthreads();                                            \
+        }
+    for(int kt = 0; kt < nkt; kt += DEPTH) {
+        NBL_FC_STEP(0, st0, st1)
+        NBL_FC_STEP(1, st1, st2)
+        NBL_FC_STEP(2, st2, st3)
+        NBL_FC_STEP(3, st3, st0)
+    }
+    #undef NBL_FC_STEP
+
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    float *__restrict__ Cout = a.C + (EPI == EPI_PARTIAL ? (size_t)blockIdx.z * a.M * a.ldc : 0);
+    const int n = n0 + wn * 32 + l32;
+    if(n >= a.N) return;
+    float gn = 1.0f, bn = 0.0f;
+    if(EPI == EPI_DIRECT) { bn = a.b[n]; if(a.has_scale) gn = a.g[n]; }
+    #pragma unroll
+    for(int i = 0; i < MT; i++)
+        #pragma unroll
+        for(int r = 0; r < 16; r++) {
+            const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            if(m >= a.M) continue;
+            float v = acc[i][r];
+            if(EPI == EPI_DIRECT) {
+                v = a.has_scale ? v * gn + bn : v + bn;
+                v = nbl_act_apply(a.act, v);
+            }
+            Cout[(size_t)m * a.ldc + n] = v;
+        }
+}
+
 // y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n])
 __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ y,
                                      const float *__restrict__ g, const float *__restrict__ b,
@@ -500,7 +627,9 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
             *ws_bytes = need;
         }
         a.C = *ws;
-        if(BM == 32)       hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((fc_stream_kernel<1, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((fc_stream_kernel<2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(split-k)");
@@ -509,7 +638,9 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
                            *ws, C, g, b, M, N, S, act, has_scale);
         NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
     } else {
-        if(BM == 32)       hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((fc_stream_kernel<1, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((fc_stream_kernel<2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel");
