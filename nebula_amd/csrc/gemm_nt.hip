@@ -213,25 +213,30 @@ void gemm_nt_kernel(const GemmArgs a) {
     }
 }
 
-// Small-batch fully connected product (M <= 64 rows): the layer is a stream of the [N][K] weight matrix
-// from HBM, so what matters is how many bytes each CU keeps in flight.  Same tiling and LDS layout as
-// gemm_nt_kernel with a 32*MT x 128 block tile, but the global loads run through a ring of four register
-// stages: while k-tile t is multiplied, tiles t+2, t+3 and t+4 are on their way (a single stage covers
-// about a quarter of the HBM latency and held the stream to 3.2 TB/s).  Every load is issued
-// unconditionally (past the end the last tile is re-read and ignored) so that the compiler waits per
-// stage, not for everything.  Output: raw partial sums part[blockIdx.z][M][N] or, with one k chunk,
-// act(sum * g + b).
-template<int MT, int EPI>
-__global__ __launch_bounds__(256)
-void fc_stream_kernel(const GemmArgs a) {
-    constexpr int BK = GEMM_BK, LD = GEMM_LD, NTHREADS = 256, DEPTH = 4;
-    constexpr int BM = MT * 32, BN = 128;
+// The same product for operands whose rows are 16-byte aligned with K % 4 == 0 (every layer of the
+// shipped networks): identical tiling and LDS layout as gemm_nt_kernel, but
+//  - every global load is an unconditional 16-byte load (a row past the matrix repeats the last row and its
+//    products are never stored; a k past the chunk re-reads the chunk's last four values and is replaced by
+//    zeros when the stage is written to LDS), so no branch makes the compiler wait for all loads at once;
+//  - the loads run through a ring of DEPTH register stages: while k-tile t is multiplied, tiles t+2 ..
+//    t+DEPTH are on their way.  At small batch (M <= 64, DEPTH = 4) the layer is a stream of the [N][K]
+//    weight matrix and the bytes in flight per CU decide its rate (one stage covers about a quarter of the
+//    HBM latency and held the stream to 3.2 TB/s); large tiles take DEPTH = 2.
+// Output: raw partial sums part[blockIdx.z][M][N] (EPI_PARTIAL) or act(sum * g + b) (EPI_DIRECT).
+template<int MT, int NT, int WAVES_M, int WAVES_N, int DEPTH, int EPI>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N)
+void gemm_nt_stream_kernel(const GemmArgs a) {
+    constexpr int BK = GEMM_BK, LD = GEMM_LD, NTHREADS = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = MT * 32 * WAVES_M, BN = NT * 32 * WAVES_N;
+    static_assert((BM * 8) % NTHREADS == 0 && (BN * 8) % NTHREADS == 0, "tiles must split evenly over the threads");
+    static_assert(DEPTH == 2 || DEPTH == 4, "the ring below is written out for two or four stages");
     constexpr int RA = BM * 8 / NTHREADS, RB = BN * 8 / NTHREADS;
     __shared__ __attribute__((aligned(16))) float As[2][BM][LD];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][LD];
-    const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     const int half = lane >> 5, l32 = lane & 31;
-    const int n0 = blockIdx.x * BN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int k_begin = blockIdx.z * a.k_chunk;
     const int k_end = min(a.K, k_begin + a.k_chunk);
     const int nkt = (k_end - k_begin + BK - 1) / BK;
@@ -239,15 +244,11 @@ void fc_stream_kernel(const GemmArgs a) {
 
     struct Stage { float4 a[RA], b[RB]; bool valid; };
     Stage st0, st1, st2, st3;           // named, not an array: an indexed array of stages ends up in scratch memory
-    static_assert(DEPTH == 4, "the ring below is written out for four stages");
-    // Unconditional 16-byte loads (rows 16-byte aligned, K % 4 == 0): a row past the matrix repeats the last
-    // row (its products are never stored), a k past the chunk re-reads the chunk's last four values and is
-    // replaced by zeros; no branch, so nothing makes the compiler wait for more than the stage it needs.
     const int acol = (tid & 7) * 4;
     const float *__restrict__ arow[RA];
     const float *__restrict__ brow[RB];
     #pragma unroll
-    for(int r = 0; r < RA; r++) arow[r] = a.A + (size_t)min((tid + r * NTHREADS) >> 3, a.M - 1) * a.lda;
+    for(int r = 0; r < RA; r++) arow[r] = a.A + (size_t)min(m0 + ((tid + r * NTHREADS) >> 3), a.M - 1) * a.lda;
     #pragma unroll
     for(int r = 0; r < RB; r++) brow[r] = a.Bw + (size_t)min(n0 + ((tid + r * NTHREADS) >> 3), a.N - 1) * a.ldb;
     auto load_tile = [&](Stage &s, int kt) {
@@ -278,66 +279,84 @@ void fc_stream_kernel(const GemmArgs a) {
                 make_float4(s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f);
         }
     };
-    floatx16 acc[MT];
+    floatx16 acc[MT][NT];
     #pragma unroll
     for(int i = 0; i < MT; i++)
         #pragma unroll
-        for(int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+        for(int j = 0; j < NT; j++)
+            #pragma unroll
+            for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
     auto compute_tile = [&](int buf) {
         #pragma unroll
         for(int q = 0; q < 4; q++) {
-            const float4 bv = *reinterpret_cast<const float4*>(&Bs[buf][wn * 32 + l32][half * 16 + q * 4]);
+            float4 av[MT], bv[NT];
             #pragma unroll
-            for(int i = 0; i < MT; i++) {
-                const float4 av = *reinterpret_cast<const float4*>(&As[buf][i * 32 + l32][half * 16 + q * 4]);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc[i], 0, 0, 0);
-            }
+            for(int i = 0; i < MT; i++)
+                av[i] = *reinterpret_cast<const float4*>(&As[buf][(wm * MT + i) * 32 + l32][half * 16 + q * 4]);
+            #pragma unroll
+            for(int j = 0; j < NT; j++)
+                bv[j] = *reinterpret_cast<const float4*>(&Bs[buf][(wn * NT + j) * 32 + l32][half * 16 + q * 4]);
+            #pragma unroll
+            for(int i = 0; i < MT; i++)
+                #pragma unroll
+                for(int j = 0; j < NT; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].x, bv[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].y, bv[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].z, bv[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i].w, bv[j].w, acc[i][j], 0, 0, 0);
+                }
         }
     };
 
-    load_tile(st0, 0); load_tile(st1, 1); load_tile(st2, 2); load_tile(st3, 3);
-    store_tile(st0, 0);
-    __syncthreads();
-    // k-tile t travels through stage t % 4 into LDS buffer t % 2.  One step: refill the stage that was written
-    // to LDS one step ago with tile t+4, multiply tile t, write tile t+1 (past the end: a repeat of the last
-    // tile, never multiplied) into the other buffer.
-    #define NBL_FC_STEP(U, CUR, NEXT)                                   \
+    // k-tile t travels through stage t % DEPTH into LDS buffer t % 2.  One step: refill the stage that was
+    // written to LDS one step ago with tile t+DEPTH, multiply tile t, write tile t+1 (past the end: a repeat of
+    // the last tile, never multiplied) into the other buffer.
+    #define NBL_GEMM_STEP(U, CUR, NEXT)                                 \
         if(kt + U < nkt) {                                              \
             load_tile(CUR, kt + U + DEPTH);                             \
             compute_tile(U & 1);                                        \
             store_tile(NEXT, (U + 1) & 1);                              \
             __syncthreads();                                            \
         }
+    load_tile(st0, 0); load_tile(st1, 1);
+    if(DEPTH == 4) { load_tile(st2, 2); load_tile(st3, 3); }
+    store_tile(st0, 0);
+    __syncthreads();
     for(int kt = 0; kt < nkt; kt += DEPTH) {
-        NBL_FC_STEP(0, st0, st1)
-        NBL_FC_STEP(1, st1, st2)
-        NBL_FC_STEP(2, st2, st3)
-        NBL_FC_STEP(3, st3, st0)
+        if(DEPTH == 4) {
+            NBL_GEMM_STEP(0, st0, st1)
+            NBL_GEMM_STEP(1, st1, st2)
+            NBL_GEMM_STEP(2, st2, st3)
+            NBL_GEMM_STEP(3, st3, st0)
+        } else {
+            NBL_GEMM_STEP(0, st0, st1)
+            NBL_GEMM_STEP(1, st1, st0)
+        }
     }
-    #undef NBL_FC_STEP
+    #undef NBL_GEMM_STEP
 
     // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
     float *__restrict__ Cout = a.C + (EPI == EPI_PARTIAL ? (size_t)blockIdx.z * a.M * a.ldc : 0);
-    const int n = n0 + wn * 32 + l32;
-    if(n >= a.N) return;
-    float gn = 1.0f, bn = 0.0f;
-    if(EPI == EPI_DIRECT) { bn = a.b[n]; if(a.has_scale) gn = a.g[n]; }
     #pragma unroll
-    for(int i = 0; i < MT; i++)
+    for(int j = 0; j < NT; j++) {
+        const int n = n0 + (wn * NT + j) * 32 + l32;
+        if(n >= a.N) continue;
+        float gn = 1.0f, bn = 0.0f;
+        if(EPI == EPI_DIRECT) { bn = a.b[n]; if(a.has_scale) gn = a.g[n]; }
         #pragma unroll
-        for(int r = 0; r < 16; r++) {
-            const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-            if(m >= a.M) continue;
-            float v = acc[i][r];
-            if(EPI == EPI_DIRECT) {
-                v = a.has_scale ? v * gn + bn : v + bn;
-                v = nbl_act_apply(a.act, v);
+        for(int i = 0; i < MT; i++)
+            #pragma unroll
+            for(int r = 0; r < 16; r++) {
+                const int m = m0 + (wm * MT + i) * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                if(m >= a.M) continue;
+                float v = acc[i][j][r];
+                if(EPI == EPI_DIRECT) {
+                    v = a.has_scale ? v * gn + bn : v + bn;
+                    v = nbl_act_apply(a.act, v);
+                }
+                Cout[(size_t)m * a.ldc + n] = v;
             }
-            Cout[(size_t)m * a.ldc + n] = v;
-        }
+    }
 }
 
 // y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n])
@@ -627,8 +646,9 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
             *ws_bytes = need;
         }
         a.C = *ws;
-        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((fc_stream_kernel<1, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
-        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((fc_stream_kernel<2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
@@ -638,8 +658,9 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
                            *ws, C, g, b, M, N, S, act, has_scale);
         NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
     } else {
-        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((fc_stream_kernel<1, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
-        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((fc_stream_kernel<2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
