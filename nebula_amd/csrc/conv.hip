@@ -28,6 +28,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
+#include <algorithm>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -127,10 +128,17 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byt
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, unsigned byte_off, unsigned uniform_off) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, (int)uniform_off, 0));
 }
+__device__ __forceinline__ auto buf_load4(__amdgpu_buffer_rsrc_t r, unsigned byte_off, unsigned uniform_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, (int)uniform_off, 0);
+}
+// Native 4-float vector: staged tiles move as values (a struct float4 copy can become a memcpy through a
+// private-memory slot that is never promoted to registers).
+typedef float vec4f __attribute__((ext_vector_type(4)));
+
 // How a block gathers its slice of the patch matrix.
 enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
        GATHER_NOPAD = 1,    // padding = 0: every tap of a real pixel is inside the image
-       GATHER_1X1_VEC4 = 2, // 1x1, stride 1, padding 0, OH*OW % 4 == 0: four pixels per 16-byte load
+       GATHER_1X1_VEC4 = 2, // 1x1, stride 1, padding 0, OH*OW % 4 == 0, C % 32 == 0: four pixels per 16-byte load
        // Patch rows ordered (c / 16, i, j, c % 16) with C a multiple of the k-tile depth: a k-tile is 16
        // channels of ONE tap, so whether the tap is inside the image is decided once per pixel and k-tile (a bit of a mask
        // computed at block start), and the 16 rows differ by a uniform plane offset that travels in the
@@ -200,7 +208,6 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int ld_m0 = (tile % a.tiles_m) * BM;
     PixelCoord px;
     unsigned xoff;
-    const float *__restrict__ xpix;
     {
         const int n0 = (tile / a.tiles_m) * BN;
         // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past
@@ -210,8 +217,21 @@ void conv_igemm_kernel(const ConvArgs a) {
         px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
         // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
         xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
-        xpix = a.x + (VEC4 ? px.xbase : 0);
     }
+    // byte offsets of this thread's loads inside one k-tile's slice of the input (1x1 vector mode) and of the
+    // packed weights; the k-tile's own offset is uniform and goes into the scalar offset of the buffer loads.
+    // (A load through a 64-bit per-lane pointer costs matrix-pipe time for its address arithmetic and issue;
+    // a buffer load with a constant vector offset and a scalar k offset costs none.)
+    unsigned vec_off[VEC4 ? RB : 1];
+    if(VEC4) {
+        #pragma unroll
+        for(int r = 0; r < RB; r++) vec_off[r] = (unsigned)(px.xbase + (krow0 + r * KGROUPS) * a.OHW) * 4u;
+    }
+    const __amdgpu_buffer_rsrc_t wres = make_rsrc(a.wp, (unsigned)a.Kp * (unsigned)a.Mp * 4u);
+    const unsigned w_off0 = A_VEC >= NTHREADS || tid < A_VEC
+        ? (unsigned)((tid / (BM / 4)) * a.Mp + (tid % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
+    const unsigned w_off1 = RA > 1 && (A_VEC >= 2 * NTHREADS || tid + NTHREADS < A_VEC)
+        ? (unsigned)(((tid + NTHREADS) / (BM / 4)) * a.Mp + ((tid + NTHREADS) % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
     unsigned tapmask = 0;       // tap-major: bit i*ksize+j set when that tap of this thread's pixel is inside the image
     if(TAPM) {
         int t = 0;
@@ -224,9 +244,8 @@ void conv_igemm_kernel(const ConvArgs a) {
     // still in flight, so every global load has two k-tiles of MFMA time to arrive.
     struct Stage {
         float b[VEC4 ? 1 : RB];
-        float4 b4[VEC4 ? RB : 1];
-        float4 a0, a1;
-        unsigned kvalid;
+        vec4f b4[VEC4 ? RB : 1];
+        vec4f a0, a1;
     };
     Stage st0, st1;
     int2 ke[VEC4 || TAPM ? 1 : RB];  // table entries of the next k-tile to gather (tap-major: the k-tile's one entry)
@@ -242,14 +261,12 @@ void conv_igemm_kernel(const ConvArgs a) {
     };
     auto load_tile = [&](Stage &st, int kt) {
         if(VEC4) {
-            st.kvalid = 0;
+            // 1x1: input plane = output plane, patch row k = channel k, and C is a multiple of 32 (no padding
+            // rows).  The k-tile's offset is uniform and travels in the scalar offset of the buffer load, the
+            // thread's own offset is constant: no vector arithmetic per load.
+            const unsigned xk = (unsigned)kt * (unsigned)(BK * sizeof(float)) * (unsigned)a.OHW;
             #pragma unroll
-            for(int r = 0; r < RB; r++) {
-                const int k = kt * BK + krow0 + r * KGROUPS;
-                st.kvalid |= (k < a.K ? 1u : 0u) << r;
-                // 1x1: input plane = output plane
-                st.b4[r] = *reinterpret_cast<const float4*>(xpix + (size_t)min(k, a.K - 1) * a.OHW);
-            }
+            for(int r = 0; r < RB; r++) st.b4[r] = __builtin_bit_cast(vec4f, buf_load4(xres, vec_off[r], xk));
         } else if(TAPM) {
             const bool inside = ke[0].y >= 0 && ((tapmask >> (ke[0].y & 31)) & 1u) != 0;
             const unsigned off = inside ? xoff + (unsigned)ke[0].x : OOB_OFFSET;   // stays out of range when xoff is
@@ -264,18 +281,11 @@ void conv_igemm_kernel(const ConvArgs a) {
                 st.b[r] = buf_load(xres, off);
             }
         }
-        const float *__restrict__ wtile = a.wp + (size_t)kt * BK * a.Mp + ld_m0;
-        {
-            const int row = tid / (BM / 4), col4 = tid % (BM / 4);
-            if(A_VEC >= NTHREADS || tid < A_VEC)
-                st.a0 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
-        }
-        if(RA > 1) {
-            const int v = tid + NTHREADS;
-            const int row = v / (BM / 4), col4 = v % (BM / 4);
-            if(A_VEC >= 2 * NTHREADS || v < A_VEC)
-                st.a1 = *reinterpret_cast<const float4*>(wtile + (size_t)row * a.Mp + col4 * 4);
-        }
+        // weights: the k-tile's uniform offset in the scalar offset, the thread's constant offset in the vector
+        // offset (out of range for a thread with nothing to load, which then reads zeros)
+        const unsigned wk = (unsigned)kt * (unsigned)(BK * sizeof(float)) * (unsigned)a.Mp;
+        st.a0 = __builtin_bit_cast(vec4f, buf_load4(wres, w_off0, wk));
+        if(RA > 1) st.a1 = __builtin_bit_cast(vec4f, buf_load4(wres, w_off1, wk));
     };
     // issue the loads of the next k-tile; the table entries of the k-tile after it follow (the tables end
     // in all-padding tiles, so the entry after the last k-tile exists)
@@ -287,21 +297,19 @@ void conv_igemm_kernel(const ConvArgs a) {
     auto store_tile = [&](const Stage &st, int buf) {
         if(VEC4) {
             #pragma unroll
-            for(int r = 0; r < RB; r++)
-                *reinterpret_cast<float4*>(&Bs[buf][krow0 + r * KGROUPS][ncol * 4]) =
-                    ((st.kvalid >> r) & 1u) ? st.b4[r] : make_float4(0.f, 0.f, 0.f, 0.f);
+            for(int r = 0; r < RB; r++) *reinterpret_cast<vec4f*>(&Bs[buf][krow0 + r * KGROUPS][ncol * 4]) = st.b4[r];
         } else {
             #pragma unroll
             for(int r = 0; r < RB; r++) Bs[buf][krow0 + r][ncol] = st.b[r];
         }
         {
             const int row = tid / (BM / 4), col4 = tid % (BM / 4);
-            if(A_VEC >= NTHREADS || tid < A_VEC) *reinterpret_cast<float4*>(&As[buf][row][col4 * 4]) = st.a0;
+            if(A_VEC >= NTHREADS || tid < A_VEC) *reinterpret_cast<vec4f*>(&As[buf][row][col4 * 4]) = st.a0;
         }
         if(RA > 1) {
             const int v = tid + NTHREADS;
             const int row = v / (BM / 4), col4 = v % (BM / 4);
-            if(A_VEC >= 2 * NTHREADS || v < A_VEC) *reinterpret_cast<float4*>(&As[buf][row][col4 * 4]) = st.a1;
+            if(A_VEC >= 2 * NTHREADS || v < A_VEC) *reinterpret_cast<vec4f*>(&As[buf][row][col4 * 4]) = st.a1;
         }
     };
 
@@ -559,7 +567,7 @@ void conv_igemm_kernel(const ConvArgs a) {
     };
 
     // ---- pipeline start: the block's first two k-tiles ----
-    st0.a0 = st0.a1 = st1.a0 = st1.a1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    st0.a0 = st0.a1 = st1.a0 = st1.a1 = vec4f{0.f, 0.f, 0.f, 0.f};
     load_ktab(kt_begin);
     ld_next(st0);
     ld_next(st1);
@@ -910,7 +918,7 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     a.ttab = p->ttab_dev; a.ksize = (int)p->k; a.plane_bytes = p->H * p->W * 4u;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
     if(p->tap_major) gather = GATHER_TAP_MAJOR;
-    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0)
+    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 && p->K == p->Kp)
         gather = GATHER_1X1_VEC4;
     a.whole_tiles = (int)blocks; a.split = 1; a.n_start = 0; a.n_tail = 0; a.ws = NULL;
     size_t grid = blocks;
@@ -951,21 +959,17 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     return NBL_OK;
 }
 
-// Tile search on the device: every tile shape runs the real problem twice and the faster second run
-// wins.  Block-count quantisation against the number of resident blocks decides more than any static
-// rule predicts, so the shapes are measured once per (layer, batch) and the result is kept in the plan.
+// Tile search on the device: every tile shape, with and without the k-split of the last round, runs the
+// real problem and the fastest wins.  Block-count quantisation against the number of resident blocks
+// decides more than any static rule predicts, so the shapes are measured once per (layer, batch) and the
+// result is kept in the plan.
 static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
                      const ConvResidual *rs) {
-    hipEvent_t e0, e1;
-    NBL_HIP(ctx, hipEventCreate(&e0));
-    hipError_t err = hipEventCreate(&e1);
-    if(err != hipSuccess) { (void)hipEventDestroy(e0); return nbl_fail(ctx, NBL_EHIP, "hipEventCreate: %s", hipGetErrorString(err)); }
-    int best = choose_variant(p, B * p->OH * p->OW, ctx->num_cu), rc = NBL_OK;
-    bool best_split = false;
-    float best_ms = 1e30f;
-    for(int v = 0; v < NUM_VARIANTS && rc == NBL_OK; v++) {
+    struct Candidate { int variant; bool split; float ms; };
+    std::vector<Candidate> cand;
+    for(int v = 0; v < NUM_VARIANTS; v++) {
         if(nbl_div_up(p->F, VARIANTS[v].bm) * VARIANTS[v].bm > p->Mp) continue;
-        for(int split = 0; split < 2 && rc == NBL_OK; split++) {
+        for(int split = 0; split < 2; split++) {
             if(split != 0 && p->split_mode == 0) continue;
             if(split == 0 && p->split_mode == 1) continue;
             if(split != 0) {    // nothing to measure where the model splits nothing
@@ -973,18 +977,47 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
                                                 VARIANTS[v].bm, VARIANTS[v].bn, p->Kp, p->F, B * p->OH * p->OW, ctx->num_cu);
                 if(sp.split <= 1 && p->split_mode != 1) continue;
             }
-            float ms = 0.0f;
-            if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, split != 0, rs)) != NBL_OK) break;
-            if(hipEventRecord(e0, ctx->stream) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed"); break; }
-            if((rc = conv_launch(ctx, p, x_dev, y_dev, B, v, split != 0, rs)) != NBL_OK) break;
-            if(hipEventRecord(e1, ctx->stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
-               hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "event timing failed"); break; }
-            if(ms < best_ms) { best_ms = ms; best = v; best_split = split != 0; }
+            cand.push_back({ v, split != 0, 0.0f });
         }
     }
-    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    const int fallback = choose_variant(p, B * p->OH * p->OW, ctx->num_cu);
+    if(cand.empty()) { p->tuned_batch = B; p->tuned_variant = fallback; p->tuned_split = p->split_mode == 1; return NBL_OK; }
+
+    // A pass queues every candidate back to back, `reps` launches each between two events, and waits once at
+    // the end: the device never idles between candidates, so all of them are measured at the same (ramped-up)
+    // clock and with the launch gaps of steady use.  Pass 1 ranks all candidates, pass 2 repeats the best few
+    // with more launches and decides.
+    std::vector<hipEvent_t> ev(cand.size() + 1);
+    size_t made = 0;
+    int rc = NBL_OK;
+    for(; made < ev.size(); made++)
+        if(hipEventCreate(&ev[made]) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventCreate failed"); break; }
+    auto pass = [&](std::vector<Candidate> &c, int reps) -> int {
+        int r = NBL_OK;
+        // clock ramp and cache warm-up, not timed
+        for(int i = 0; i < 2 * reps && r == NBL_OK; i++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[0].variant, c[0].split, rs);
+        for(size_t i = 0; i < c.size() && r == NBL_OK; i++) {
+            if(hipEventRecord(ev[i], ctx->stream) != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed");
+            for(int k = 0; k < reps && r == NBL_OK; k++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[i].variant, c[i].split, rs);
+        }
+        if(r != NBL_OK) return r;
+        if(hipEventRecord(ev[c.size()], ctx->stream) != hipSuccess || hipEventSynchronize(ev[c.size()]) != hipSuccess)
+            return nbl_fail(ctx, NBL_EHIP, "event timing failed");
+        for(size_t i = 0; i < c.size(); i++)
+            if(hipEventElapsedTime(&c[i].ms, ev[i], ev[i + 1]) != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "hipEventElapsedTime failed");
+        return NBL_OK;
+    };
+    if(rc == NBL_OK) rc = pass(cand, 3);
+    if(rc == NBL_OK) {
+        std::sort(cand.begin(), cand.end(), [](const Candidate &l, const Candidate &r) { return l.ms < r.ms; });
+        if(cand.size() > 3) cand.resize(3);
+        rc = pass(cand, 10);
+    }
+    for(size_t i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
     if(rc != NBL_OK) return rc;
-    p->tuned_batch = B; p->tuned_variant = best; p->tuned_split = best_split;
+    size_t best = 0;
+    for(size_t i = 1; i < cand.size(); i++) if(cand[i].ms < cand[best].ms) best = i;
+    p->tuned_batch = B; p->tuned_variant = cand[best].variant; p->tuned_split = cand[best].split;
     return NBL_OK;
 }
 
