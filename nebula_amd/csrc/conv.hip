@@ -59,7 +59,8 @@ struct ConvArgs {
     int units;     // whole_tiles + (tiles - whole_tiles) * split: work units of the launch
     float *ws;
     // tap-major layers: one entry per k-tile, {byte offset of the tile's tap in channel c0's plane +
-    // c0*H*W*4, tap index i*ksize+j or -1 for an all-padding tile}
+    // c0*H*W*4, 31 - tap index (the left shift that brings the tap's bit of a pixel's outside mask to
+    // bit 31), or 0 for an all-padding tile}
     const int2 *ttab; int ksize; unsigned plane_bytes;
 };
 
@@ -232,12 +233,14 @@ void conv_igemm_kernel(const ConvArgs a) {
         ? (unsigned)((tid / (BM / 4)) * a.Mp + (tid % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
     const unsigned w_off1 = RA > 1 && (A_VEC >= 2 * NTHREADS || tid + NTHREADS < A_VEC)
         ? (unsigned)(((tid + NTHREADS) / (BM / 4)) * a.Mp + ((tid + NTHREADS) % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
-    unsigned tapmask = 0;       // tap-major: bit i*ksize+j set when that tap of this thread's pixel is inside the image
+    // tap-major: bit i*ksize+j is set when that tap of this thread's pixel is OUTSIDE the image; bit 31 is always
+    // set and stands for the padding k-tiles behind the last patch row
+    unsigned outmask = 0x80000000u;
     if(TAPM) {
         int t = 0;
         for(int i = 0; i < a.ksize; i++)
             for(int j = 0; j < a.ksize; j++, t++)
-                if((unsigned)(px.ih0 + i) < (unsigned)a.H && (unsigned)(px.iw0 + j) < (unsigned)a.W) tapmask |= 1u << t;
+                if(!((unsigned)(px.ih0 + i) < (unsigned)a.H && (unsigned)(px.iw0 + j) < (unsigned)a.W)) outmask |= 1u << t;
     }
 
     // Two register stages: the loads of k-tile t+2 are issued while k-tile t is multiplied and t+1 is
@@ -268,8 +271,9 @@ void conv_igemm_kernel(const ConvArgs a) {
             #pragma unroll
             for(int r = 0; r < RB; r++) st.b4[r] = __builtin_bit_cast(vec4f, buf_load4(xres, vec_off[r], xk));
         } else if(TAPM) {
-            const bool inside = ke[0].y >= 0 && ((tapmask >> (ke[0].y & 31)) & 1u) != 0;
-            const unsigned off = inside ? xoff + (unsigned)ke[0].x : OOB_OFFSET;   // stays out of range when xoff is
+            // the tap's bit of the outside mask, moved to bit 31, pushes the offset out of range (the pixel's own
+            // offset plus the tap's is below 2^31, or already out of range for a column past the last pixel)
+            const unsigned off = (xoff + (unsigned)ke[0].x) | ((outmask << (ke[0].y & 31)) & 0x80000000u);
             #pragma unroll
             for(int r = 0; r < RB; r++) st.b[r] = buf_load(xres, off, (unsigned)(krow0 + r) * a.plane_bytes);
         } else {
@@ -678,9 +682,9 @@ std::vector<int2> build_ttab(unsigned C, unsigned H, unsigned W, unsigned k, uns
         if(kt * CONV_BK < K) {
             const unsigned t = kt % taps, c0 = kt / taps * CONV_BK, i = t / k, j = t % k;
             tab[kt].x = (int)((c0 * H * W + i * W + j) * 4);
-            tab[kt].y = (int)t;
+            tab[kt].y = (int)(31 - t);      // shift that brings the tap's bit of the outside mask to bit 31
         } else {
-            tab[kt].x = 0; tab[kt].y = -1;
+            tab[kt].x = 0; tab[kt].y = 0;   // padding tile: bit 31 of the mask, which is always set
         }
     }
     return tab;
@@ -715,7 +719,7 @@ struct nbl_conv_plan {
     unsigned C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp;
     int act; bool has_scale;
     float *wp_dev; int2 *ktab_dev; float *g_dev; float *b_dev;
-    bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 32)
+    bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 31)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
     int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so
@@ -806,7 +810,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->split_mode = -1; p->tuned_split = false; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
-    p->tap_major = ksize > 1 && ksize * ksize <= 32 && C % CONV_BK == 0;
+    p->tap_major = ksize > 1 && ksize * ksize <= 31 && C % CONV_BK == 0;
 
     // [F][K] -> [Kp][Mp], zero padded
     std::vector<float> wp((size_t)p->Kp * p->Mp, 0.0f);
