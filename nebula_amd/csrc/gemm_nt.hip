@@ -30,6 +30,8 @@ constexpr int GEMM_LD = GEMM_BK + 4;
 
 enum { EPI_DIRECT = 0, EPI_PARTIAL = 1, EPI_LSTM = 2 };
 
+typedef float vec4f __attribute__((ext_vector_type(4)));
+
 struct GemmArgs {
     const float *A; const float *Bw; float *C;
     int M, N, K, lda, ldb, ldc;
@@ -223,7 +225,7 @@ void gemm_nt_kernel(const GemmArgs a) {
 //    weight matrix and the bytes in flight per CU decide its rate (one stage covers about a quarter of the
 //    HBM latency and held the stream to 3.2 TB/s); large tiles take DEPTH = 2.
 // Output: raw partial sums part[blockIdx.z][M][N] (EPI_PARTIAL) or act(sum * g + b) (EPI_DIRECT).
-template<int MT, int NT, int WAVES_M, int WAVES_N, int DEPTH, int EPI>
+template<int MT, int NT, int WAVES_M, int WAVES_N, int DEPTH, int EPI, bool BUF>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N)
 void gemm_nt_stream_kernel(const GemmArgs a) {
     constexpr int BK = GEMM_BK, LD = GEMM_LD, NTHREADS = 64 * WAVES_M * WAVES_N;
@@ -242,41 +244,69 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
     const int nkt = (k_end - k_begin + BK - 1) / BK;
     if(nkt <= 0) return;
 
-    struct Stage { float4 a[RA], b[RB]; bool valid; };
+    struct Stage { vec4f a[RA], b[RB]; bool valid; };
     Stage st0, st1, st2, st3;           // named, not an array: an indexed array of stages ends up in scratch memory
     const int acol = (tid & 7) * 4;
     const float *__restrict__ arow[RA];
     const float *__restrict__ brow[RB];
-    #pragma unroll
-    for(int r = 0; r < RA; r++) arow[r] = a.A + (size_t)min(m0 + ((tid + r * NTHREADS) >> 3), a.M - 1) * a.lda;
-    #pragma unroll
-    for(int r = 0; r < RB; r++) brow[r] = a.Bw + (size_t)min(n0 + ((tid + r * NTHREADS) >> 3), a.N - 1) * a.ldb;
+    // BUF (every k-tile whole, operands below 2 GiB): buffer loads whose vector offset is the thread's constant
+    // (row, column) offset -- out of range for a row past the matrix, which then reads zeros -- and whose scalar
+    // offset is the k-tile's: no vector arithmetic per load and nothing to zero afterwards.
+    unsigned aoff[RA], boff[RB];
+    __amdgpu_buffer_rsrc_t ares, bres;
+    if(BUF) {
+        ares = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.A), 0, (int)((unsigned)a.M * (unsigned)a.lda * 4u), 0x00020000);
+        bres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.Bw), 0, (int)((unsigned)a.N * (unsigned)a.ldb * 4u), 0x00020000);
+        #pragma unroll
+        for(int r = 0; r < RA; r++) {
+            const int row = m0 + ((tid + r * NTHREADS) >> 3);
+            aoff[r] = row < a.M ? ((unsigned)row * (unsigned)a.lda + (unsigned)acol) * 4u : 0x80000000u;
+        }
+        #pragma unroll
+        for(int r = 0; r < RB; r++) {
+            const int row = n0 + ((tid + r * NTHREADS) >> 3);
+            boff[r] = row < a.N ? ((unsigned)row * (unsigned)a.ldb + (unsigned)acol) * 4u : 0x80000000u;
+        }
+    } else {
+        #pragma unroll
+        for(int r = 0; r < RA; r++) arow[r] = a.A + (size_t)min(m0 + ((tid + r * NTHREADS) >> 3), a.M - 1) * a.lda;
+        #pragma unroll
+        for(int r = 0; r < RB; r++) brow[r] = a.Bw + (size_t)min(n0 + ((tid + r * NTHREADS) >> 3), a.N - 1) * a.ldb;
+    }
     auto load_tile = [&](Stage &s, int kt) {
+        if(BUF) {
+            const unsigned ko = (unsigned)(k_begin + min(kt, nkt - 1) * BK) * 4u;     // uniform
+            s.valid = true;
+            #pragma unroll
+            for(int r = 0; r < RA; r++) s.a[r] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(ares, (int)aoff[r], (int)ko, 0));
+            #pragma unroll
+            for(int r = 0; r < RB; r++) s.b[r] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(bres, (int)boff[r], (int)ko, 0));
+            return;
+        }
         const int k = k_begin + min(kt, nkt - 1) * BK + acol;
         const bool valid = k < k_end;
         const int kk = valid ? k : k_end - 4;
         s.valid = valid;            // the zeroing happens when the stage is written to LDS: touching the values
                                     // here would make the loads wait for themselves
         #pragma unroll
-        for(int r = 0; r < RA; r++) s.a[r] = *reinterpret_cast<const float4*>(arow[r] + kk);
+        for(int r = 0; r < RA; r++) s.a[r] = *reinterpret_cast<const vec4f*>(arow[r] + kk);
         #pragma unroll
-        for(int r = 0; r < RB; r++) s.b[r] = *reinterpret_cast<const float4*>(brow[r] + kk);
+        for(int r = 0; r < RB; r++) s.b[r] = *reinterpret_cast<const vec4f*>(brow[r] + kk);
     };
-    // (component-wise selects: a select between two whole float4 objects is compiled through scratch memory)
     auto store_tile = [&](const Stage &s, int buf) {
         #pragma unroll
         for(int r = 0; r < RA; r++) {
             const int v = tid + r * NTHREADS;
-            const float4 t = s.a[r];
-            *reinterpret_cast<float4*>(&As[buf][v >> 3][(v & 7) * 4]) =
-                make_float4(s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f);
+            const vec4f t = s.a[r];
+            *reinterpret_cast<vec4f*>(&As[buf][v >> 3][(v & 7) * 4]) =
+                BUF ? t : vec4f{s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f};
         }
         #pragma unroll
         for(int r = 0; r < RB; r++) {
             const int v = tid + r * NTHREADS;
-            const float4 t = s.b[r];
-            *reinterpret_cast<float4*>(&Bs[buf][v >> 3][(v & 7) * 4]) =
-                make_float4(s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f);
+            const vec4f t = s.b[r];
+            *reinterpret_cast<vec4f*>(&Bs[buf][v >> 3][(v & 7) * 4]) =
+                BUF ? t : vec4f{s.valid ? t.x : 0.f, s.valid ? t.y : 0.f, s.valid ? t.z : 0.f, s.valid ? t.w : 0.f};
         }
     };
     floatx16 acc[MT][NT];
@@ -312,7 +342,7 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
     // written to LDS one step ago with tile t+DEPTH, multiply tile t, write tile t+1 (past the end: a repeat of
     // the last tile, never multiplied) into the other buffer.
     #define NBL_GEMM_STEP(U, CUR, NEXT)                                 \
-        if(kt + U < nkt) {                                              \
+        {                                                               \
             load_tile(CUR, kt + U + DEPTH);                             \
             compute_tile(U & 1);                                        \
             store_tile(NEXT, (U + 1) & 1);                              \
@@ -322,7 +352,10 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
     if(DEPTH == 4) { load_tile(st2, 2); load_tile(st3, 3); }
     store_tile(st0, 0);
     __syncthreads();
-    for(int kt = 0; kt < nkt; kt += DEPTH) {
+    // whole rounds of the ring run without a condition inside (a conditional step makes the compiler wait for
+    // nearly every outstanding load where the paths join); the last nkt % DEPTH tiles follow one by one
+    int kt = 0;
+    for(; kt + DEPTH <= nkt; kt += DEPTH) {
         if(DEPTH == 4) {
             NBL_GEMM_STEP(0, st0, st1)
             NBL_GEMM_STEP(1, st1, st2)
@@ -332,6 +365,11 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
             NBL_GEMM_STEP(0, st0, st1)
             NBL_GEMM_STEP(1, st1, st0)
         }
+    }
+    if(kt < nkt) NBL_GEMM_STEP(0, st0, st1)
+    if(DEPTH == 4) {
+        if(kt + 1 < nkt) NBL_GEMM_STEP(1, st1, st2)
+        if(kt + 2 < nkt) NBL_GEMM_STEP(2, st2, st3)
     }
     #undef NBL_GEMM_STEP
 
@@ -359,18 +397,41 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
     }
 }
 
-// y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n])
+// y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n]), the parts added in ascending z.  VEC adjacent n per thread
+// (VEC = 4 needs N % 4 == 0 and 16-byte aligned buffers); eight parts are requested before the first is added, so
+// the kernel is one memory round trip per eight parts instead of one per part.
+template<int VEC>
 __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ y,
                                      const float *__restrict__ g, const float *__restrict__ b,
                                      int M, int N, int S, int act, int has_scale) {
-    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    typedef float __attribute__((ext_vector_type(VEC))) vec;
+    const size_t e = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     const size_t total = (size_t)M * N;
     if(e >= total) return;
     const int n = (int)(e % N);
-    float v = 0.0f;
-    for(int z = 0; z < S; z++) v += part[(size_t)z * total + e];
-    v = has_scale ? v * g[n] + b[n] : v + b[n];
-    y[e] = nbl_act_apply(act, v);
+    vec v = 0.0f;
+    int z = 0;
+    for(; z + 8 <= S; z += 8) {
+        vec t[8];
+        #pragma unroll
+        for(int u = 0; u < 8; u++) t[u] = *reinterpret_cast<const vec*>(part + (size_t)(z + u) * total + e);
+        #pragma unroll
+        for(int u = 0; u < 8; u++)
+            #pragma unroll
+            for(int c = 0; c < VEC; c++) v[c] = __fadd_rn(v[c], t[u][c]);
+    }
+    for(; z < S; z++) {
+        const vec t = *reinterpret_cast<const vec*>(part + (size_t)z * total + e);
+        #pragma unroll
+        for(int c = 0; c < VEC; c++) v[c] = __fadd_rn(v[c], t[c]);
+    }
+    vec o;
+    #pragma unroll
+    for(int c = 0; c < VEC; c++) {
+        const float s = has_scale ? v[c] * g[n + c] + b[n + c] : v[c] + b[n + c];
+        o[c] = nbl_act_apply(act, s);
+    }
+    *reinterpret_cast<vec*>(y + e) = o;
 }
 
 // A wave's share of a skinny product: acc0 + acc1 = sum over `kw` consecutive k of A[row][k] * B[col][k]
@@ -636,6 +697,8 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     a.k_chunk = nbl_div_up(ktiles, S) * GEMM_BK;
     S = nbl_div_up(K, a.k_chunk);
     dim3 grid(gn, gm, S), block(256);
+    // every k-tile whole and both operands addressable by 31-bit byte offsets: the buffer-load variant
+    const bool buf_ok = a.vec_ok && K % GEMM_BK == 0 && (size_t)M * K * 4 < (1ull << 31) && (size_t)N * K * 4 < (1ull << 31);
     if(S > 1) {
         const size_t need = (size_t)S * M * N * sizeof(float);
         if(*ws_bytes < need) {
@@ -646,21 +709,31 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
             *ws_bytes = need;
         }
         a.C = *ws;
-        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
-        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
-        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
+        else if(buf_ok)                hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, false>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL, false>), grid, block, 0, ctx->stream, a);
+        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL, false>), grid, block, 0, ctx->stream, a);
         else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(split-k)");
         const size_t total = (size_t)M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
-                           *ws, C, g, b, M, N, S, act, has_scale);
+        if(N % 4 == 0 && aligned16(*ws) && aligned16(C))
+            hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
+                               *ws, C, g, b, M, N, S, act, has_scale);
+        else
+            hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                               *ws, C, g, b, M, N, S, act, has_scale);
         NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
     } else {
-        if(BM == 32 && a.vec_ok)       hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
-        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
-        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
+        if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
+        else if(buf_ok)                hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, false>), grid, block, 0, ctx->stream, a);
+        else if(BM == 64 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT, false>), grid, block, 0, ctx->stream, a);
+        else if(a.vec_ok)              hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_DIRECT, false>), grid, block, 0, ctx->stream, a);
         else if(BM == 32)  hipLaunchKernelGGL((gemm_nt_kernel<1, 1, 1, 4, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_DIRECT>), grid, block, 0, ctx->stream, a);
