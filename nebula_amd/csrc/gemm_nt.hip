@@ -690,7 +690,7 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     // Split K so that every CU walks about the same number of k-tiles: blocks are dealt to the CUs round robin, so a
     // launch lasts as long as the CU with the most blocks, ceil(blocks / CUs) chunks of k-tiles plus a partial tile
     // written (and read again by the reduction) per block.  The chunk count need not be a power of two: 640 blocks on
-    // 256 CUs stream 17 % slower than 760.
+    // 256 CUs (three on some, two on others) stream a 492 MB matrix 7 % slower than 500.
     int S = 1;
     const int ktiles = nbl_div_up(K, GEMM_BK);
     if(ws) {
