@@ -114,7 +114,8 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
  * the unsplit sum order).  A plan keeps the scratch memory for this, so one plan must not run on two
  * streams at once.  mode -1 (default): measured
  * together with the tile shape on the first call at a batch size; 0: never; 1: wherever the built-in
- * cost model says so.  No counterpart in the reference, whose GEMM is cuBLAS's choice
+ * cost model says so, with its slice count; 2..8: always, with that many slices (fewer where the patch
+ * rows run out).  No counterpart in the reference, whose GEMM is cuBLAS's choice
  * (models/layers/convolutional_layer.cu:53-74). */
 int nbl_conv2d_plan_set_split(nbl_conv_plan *plan, int mode);
 /* Tile shape (index below nbl_conv2d_num_variants(), -1 before the first call) and number of k slices

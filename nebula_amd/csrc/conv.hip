@@ -606,37 +606,49 @@ void conv_igemm_kernel(const ConvArgs a) {
 }
 
 // Second half of a k-split convolution: adds the parts in order and applies the epilogue the whole-tile
-// blocks apply themselves.  One thread per filter and VEC adjacent pixel columns of the split region;
-// VEC = 4 needs OH*OW and the region's width to be multiples of 4, so that a thread's pixels are one
-// aligned vector of one output plane.
-template<int VEC>
+// blocks apply themselves.  One thread per filter and VEC adjacent pixel columns of the split region (VEC = 4
+// needs the region's width to be a multiple of 4).  All parts are requested before the first is added -- there are
+// at most 8, and a part index past the count re-reads the last part instead of branching -- so the kernel is one
+// memory round trip, not one per part.  VSTORE: the thread's pixels are one aligned vector of one output plane
+// (OH*OW % 4 == 0); otherwise each pixel finds its own place.
+template<int VEC, bool VSTORE>
 __global__ void conv_split_finish_kernel(const ConvArgs a) {
     typedef float __attribute__((ext_vector_type(VEC))) vec;
     const int nloc = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     const int f = blockIdx.y;
     if(nloc >= a.n_tail) return;
     const size_t part_elems = (size_t)a.F * a.n_tail, at = (size_t)f * a.n_tail + nloc;
-    vec t = *reinterpret_cast<const vec*>(a.ws + at);
-    for(int p = 1; p < a.split; p++) {
-        const vec u = *reinterpret_cast<const vec*>(a.ws + p * part_elems + at);
-        #pragma unroll
-        for(int e = 0; e < VEC; e++) t[e] = __fadd_rn(t[e], u[e]);
+    vec part[8];
+    #pragma unroll
+    for(int p = 0; p < 8; p++) part[p] = *reinterpret_cast<const vec*>(a.ws + (size_t)min(p, a.split - 1) * part_elems + at);
+    vec t = part[0];
+    #pragma unroll
+    for(int p = 1; p < 8; p++) {
+        if(p < a.split) {
+            #pragma unroll
+            for(int e = 0; e < VEC; e++) t[e] = __fadd_rn(t[e], part[p][e]);
+        }
     }
     const float g = a.g[f], bias = a.b[f];
-    const int n = a.n_start + nloc;
-    const int b = n / a.OHW, pix = n - b * a.OHW;
+    const int n0 = a.n_start + nloc;
+    int b = n0 / a.OHW, pix = n0 - b * a.OHW;
     #pragma unroll
     for(int e = 0; e < VEC; e++) {
         float v = nbl_act_apply(a.act, __builtin_fmaf(t[e], g, bias));
         if(a.res) {
-            const int h = (pix + e) / a.OW, w = (pix + e) - h * a.OW;
+            const int h = pix / a.OW, w = pix - h * a.OW;
             if(f < a.res_c && h < a.res_box_h && w < a.res_box_w)
                 v = __fadd_rn(v, a.res[((size_t)b * a.res_c + f) * a.res_hw + h * a.res_stride * a.res_w + w * a.res_stride]);
             v = nbl_act_apply(a.post_act, v);
         }
-        t[e] = v;
+        if(VSTORE) t[e] = v;
+        else a.y[((size_t)b * a.F + f) * a.OHW + pix] = v;
+        if(++pix == a.OHW) { pix = 0; ++b; }       // the next pixel may belong to the next image
     }
-    *reinterpret_cast<vec*>(a.y + ((size_t)b * a.F + f) * a.OHW + pix) = t;
+    if(VSTORE) {
+        b = n0 / a.OHW; pix = n0 - b * a.OHW;
+        *reinterpret_cast<vec*>(a.y + ((size_t)b * a.F + f) * a.OHW + pix) = t;
+    }
 }
 
 __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restrict__ ktab, float *__restrict__ col,
@@ -722,8 +734,8 @@ struct nbl_conv_plan {
     bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 31)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
-    int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so
-    bool tuned_split;
+    int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so, 2..8 always with that many slices
+    int tuned_slices;           // 0 = unsplit, 1 = the cost model's slice count, 2..8 = that many
     float *ws_dev; size_t ws_bytes;   // partial sums of split launches (grown on demand)
     int last_variant, last_split;     // what the most recent launch used
 };
@@ -755,7 +767,8 @@ int choose_variant(const nbl_conv_plan *p, unsigned N, int num_cu) {
 // over the idle CUs; the price is writing and re-reading the partial sums and one more small launch.
 struct SplitPlan { int whole_tiles, split; };
 
-SplitPlan plan_split(int tiles_m, int tiles_n, int bm, int bn, unsigned Kp, unsigned F, unsigned N, int num_cu) {
+// forced: 0 = the cost model chooses the slice count, 2..8 = that many slices (fewer if the patch rows run out)
+SplitPlan plan_split(int tiles_m, int tiles_n, int bm, int bn, unsigned Kp, unsigned F, unsigned N, int num_cu, int forced = 0) {
     const int tiles = tiles_m * tiles_n, pairs = (int)(Kp / (2 * CONV_BK));
     SplitPlan none = { tiles, 1 };
     int whole = tiles / num_cu * num_cu;
@@ -771,6 +784,10 @@ SplitPlan plan_split(int tiles_m, int tiles_n, int bm, int bn, unsigned Kp, unsi
         if(ws_bytes > ((size_t)1 << 30)) break;
         const double us = std::ceil((double)left * g / num_cu) / g * tile_us + 2.0 * ws_bytes / 4e12 * 1e6 + 5.0;
         if(us < best_us) { best_us = us; best = g; }
+    }
+    if(forced >= 2) {
+        best = forced < pairs ? forced : pairs;
+        if((size_t)best * F * n_tail * sizeof(float) > ((size_t)1 << 30)) return none;
     }
     if(best == 1) return none;
     SplitPlan sp = { whole, best };
@@ -807,7 +824,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->Kp = nbl_div_up(p->K, 2 * CONV_BK) * 2 * CONV_BK;   // the k loop consumes tiles in pairs
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
-    p->split_mode = -1; p->tuned_split = false; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
+    p->split_mode = -1; p->tuned_slices = 0; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
     p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
     p->tap_major = ksize > 1 && ksize * ksize <= 31 && C % CONV_BK == 0;
@@ -867,7 +884,7 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
 }
 
 int nbl_conv2d_plan_set_split(nbl_conv_plan *p, int mode) {
-    if(!p || mode < -1 || mode > 1) return NBL_EINVAL;
+    if(!p || mode < -1 || mode > 8) return NBL_EINVAL;
     p->split_mode = mode;
     p->tuned_batch = 0;     // the next call searches again under the new rule
     return NBL_OK;
@@ -882,8 +899,9 @@ int nbl_conv2d_plan_last_launch(const nbl_conv_plan *p, int *variant, int *split
 
 struct ConvResidual { const float *res; unsigned c, h, w; int post_act; };
 
+// slices: 0 = unsplit, 1 = k-split with the cost model's slice count, 2..8 = k-split with that many slices
 static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v,
-                       bool split, const ConvResidual *rs) {
+                       int slices, const ConvResidual *rs) {
     const size_t in_elems = (size_t)B * p->C * p->H * p->W;
     const size_t npix = (size_t)B * p->OH * p->OW;
     const Variant &var = VARIANTS[v];
@@ -926,8 +944,9 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
         gather = GATHER_1X1_VEC4;
     a.whole_tiles = (int)blocks; a.split = 1; a.n_start = 0; a.n_tail = 0; a.ws = NULL;
     size_t grid = blocks;
-    if(split && p->F <= 65535) {      // the finishing kernel's grid has one row per filter
-        const SplitPlan sp = plan_split(a.tiles_m, a.tiles_n, var.bm, var.bn, p->Kp, p->F, (unsigned)npix, ctx->num_cu);
+    if(slices && p->F <= 65535) {     // the finishing kernel's grid has one row per filter
+        const SplitPlan sp = plan_split(a.tiles_m, a.tiles_n, var.bm, var.bn, p->Kp, p->F, (unsigned)npix, ctx->num_cu,
+                                        slices >= 2 ? slices : 0);
         if(sp.split > 1) {
             a.whole_tiles = sp.whole_tiles; a.split = sp.split;
             a.n_start = sp.whole_tiles / a.tiles_m * var.bn;
@@ -953,10 +972,13 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     p->last_variant = v; p->last_split = a.split;
     if(a.split > 1) {
         if(a.OHW % 4 == 0 && a.n_tail % 4 == 0 && ((size_t)y_dev & 15) == 0)
-            hipLaunchKernelGGL(conv_split_finish_kernel<4>, dim3(nbl_div_up((unsigned)a.n_tail / 4, 256), p->F), dim3(256), 0,
+            hipLaunchKernelGGL((conv_split_finish_kernel<4, true>), dim3(nbl_div_up((unsigned)a.n_tail / 4, 256), p->F), dim3(256), 0,
+                               ctx->stream, a);
+        else if(a.n_tail % 4 == 0)
+            hipLaunchKernelGGL((conv_split_finish_kernel<4, false>), dim3(nbl_div_up((unsigned)a.n_tail / 4, 256), p->F), dim3(256), 0,
                                ctx->stream, a);
         else
-            hipLaunchKernelGGL(conv_split_finish_kernel<1>, dim3(nbl_div_up((unsigned)a.n_tail, 256), p->F), dim3(256), 0,
+            hipLaunchKernelGGL((conv_split_finish_kernel<1, false>), dim3(nbl_div_up((unsigned)a.n_tail, 256), p->F), dim3(256), 0,
                                ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "conv_split_finish_kernel");
     }
@@ -969,27 +991,26 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
 // result is kept in the plan.
 static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
                      const ConvResidual *rs) {
-    struct Candidate { int variant; bool split; float ms; };
+    struct Candidate { int variant; int slices; float ms; };
     std::vector<Candidate> cand;
     for(int v = 0; v < NUM_VARIANTS; v++) {
         if(nbl_div_up(p->F, VARIANTS[v].bm) * VARIANTS[v].bm > p->Mp) continue;
-        for(int split = 0; split < 2; split++) {
-            if(split != 0 && p->split_mode == 0) continue;
-            if(split == 0 && p->split_mode == 1) continue;
-            if(split != 0) {    // nothing to measure where the model splits nothing
-                const SplitPlan sp = plan_split(nbl_div_up(p->F, VARIANTS[v].bm), nbl_div_up(B * p->OH * p->OW, VARIANTS[v].bn),
-                                                VARIANTS[v].bm, VARIANTS[v].bn, p->Kp, p->F, B * p->OH * p->OW, ctx->num_cu);
-                if(sp.split <= 1 && p->split_mode != 1) continue;
-            }
-            cand.push_back({ v, split != 0, 0.0f });
+        if(p->split_mode <= 0) cand.push_back({ v, 0, 0.0f });
+        if(p->split_mode != 0) {
+            const int slices = p->split_mode >= 2 ? p->split_mode : 1;
+            const SplitPlan sp = plan_split(nbl_div_up(p->F, VARIANTS[v].bm), nbl_div_up(B * p->OH * p->OW, VARIANTS[v].bn),
+                                            VARIANTS[v].bm, VARIANTS[v].bn, p->Kp, p->F, B * p->OH * p->OW, ctx->num_cu,
+                                            slices >= 2 ? slices : 0);
+            // nothing to measure where nothing is split (but a launch must exist when the caller insists on splitting)
+            if(sp.split > 1 || p->split_mode > 0) cand.push_back({ v, slices, 0.0f });
         }
     }
     const int fallback = choose_variant(p, B * p->OH * p->OW, ctx->num_cu);
-    if(cand.empty()) { p->tuned_batch = B; p->tuned_variant = fallback; p->tuned_split = p->split_mode == 1; return NBL_OK; }
+    if(cand.empty()) { p->tuned_batch = B; p->tuned_variant = fallback; p->tuned_slices = p->split_mode > 0 ? p->split_mode : 0; return NBL_OK; }
 
     // A pass queues every candidate back to back, `reps` launches each between two events, and waits once at
     // the end: the device never idles between candidates, so all of them are measured at the same (ramped-up)
-    // clock and with the launch gaps of steady use.  Pass 1 ranks all candidates, pass 2 repeats the best few
+    // clock and with the launch gaps of steady use.  Pass 1 ranks all candidates, pass 2 repeats the best four
     // with more launches and decides.
     std::vector<hipEvent_t> ev(cand.size() + 1);
     size_t made = 0;
@@ -999,10 +1020,10 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
     auto pass = [&](std::vector<Candidate> &c, int reps) -> int {
         int r = NBL_OK;
         // clock ramp and cache warm-up, not timed
-        for(int i = 0; i < 2 * reps && r == NBL_OK; i++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[0].variant, c[0].split, rs);
+        for(int i = 0; i < 2 * reps && r == NBL_OK; i++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[0].variant, c[0].slices, rs);
         for(size_t i = 0; i < c.size() && r == NBL_OK; i++) {
             if(hipEventRecord(ev[i], ctx->stream) != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "hipEventRecord failed");
-            for(int k = 0; k < reps && r == NBL_OK; k++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[i].variant, c[i].split, rs);
+            for(int k = 0; k < reps && r == NBL_OK; k++) r = conv_launch(ctx, p, x_dev, y_dev, B, c[i].variant, c[i].slices, rs);
         }
         if(r != NBL_OK) return r;
         if(hipEventRecord(ev[c.size()], ctx->stream) != hipSuccess || hipEventSynchronize(ev[c.size()]) != hipSuccess)
@@ -1011,17 +1032,17 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
             if(hipEventElapsedTime(&c[i].ms, ev[i], ev[i + 1]) != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "hipEventElapsedTime failed");
         return NBL_OK;
     };
-    if(rc == NBL_OK) rc = pass(cand, 3);
+    if(rc == NBL_OK) rc = pass(cand, 5);
     if(rc == NBL_OK) {
         std::sort(cand.begin(), cand.end(), [](const Candidate &l, const Candidate &r) { return l.ms < r.ms; });
-        if(cand.size() > 3) cand.resize(3);
-        rc = pass(cand, 10);
+        if(cand.size() > 4) cand.resize(4);
+        rc = pass(cand, 15);
     }
     for(size_t i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
     if(rc != NBL_OK) return rc;
     size_t best = 0;
     for(size_t i = 1; i < cand.size(); i++) if(cand[i].ms < cand[best].ms) best = i;
-    p->tuned_batch = B; p->tuned_variant = cand[best].variant; p->tuned_split = cand[best].split;
+    p->tuned_batch = B; p->tuned_variant = cand[best].variant; p->tuned_slices = cand[best].slices;
     return NBL_OK;
 }
 
@@ -1033,17 +1054,17 @@ static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_
     if(in_elems >= (1ull << 29) || out_elems >= (1ull << 31) || npix >= (1ull << 31) - 512)
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: inputs of 2^29 elements (2 GiB) or more are not supported");
     int v = p->variant;
-    bool split = p->split_mode == 1;
+    int slices = p->split_mode > 0 ? p->split_mode : 0;
     if(v < 0) {
         if(p->tuned_batch != B) {
             // the search overwrites y with correct results several times; tiny problems are not worth it
-            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); p->tuned_split = p->split_mode == 1; }
+            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); p->tuned_slices = p->split_mode > 0 ? p->split_mode : 0; }
             else { int rc = conv_tune(ctx, p, x_dev, y_dev, B, rs); if(rc != NBL_OK) return rc; }
         }
         v = p->tuned_variant;
-        split = p->tuned_split;
+        slices = p->tuned_slices;
     }
-    return conv_launch(ctx, p, x_dev, y_dev, B, v, split, rs);
+    return conv_launch(ctx, p, x_dev, y_dev, B, v, slices, rs);
 }
 
 int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {

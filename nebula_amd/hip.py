@@ -348,7 +348,7 @@ class ConvPlan:
         return v.value, g.value
 
     def set_split(self, mode):
-        """-1: measured on first use, 0: never split along k, 1: split wherever the cost model says so."""
+        """-1: measured on first use, 0: never split along k, 1: split wherever the cost model says so, 2..8: that many slices."""
         self.ctx.check(lib().nbl_conv2d_plan_set_split(self.p, mode))
 
     def __call__(self, x, out=None):

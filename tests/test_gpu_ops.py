@@ -138,6 +138,14 @@ def test_conv_k_split_matches_oracle_and_unsplit(ctx, case):
         again = run()
         np.testing.assert_array_equal(bits(got), bits(again))           # fixed summation order
     assert split_seen >= 3, "the cost model was expected to split most tile shapes of %r" % (case,)
+    # a slice count chosen by hand (fewer only where the patch rows run out)
+    plan.set_variant(4)
+    for slices in (2, 3, 8):
+        announce("conv forced slices", slices)
+        plan.set_split(slices)
+        got = run()
+        assert 1 <= plan.last_launch()[1] <= slices
+        assert rel(got, want) <= TOL, (case, slices, rel(got, want))
     plan.set_variant(-1)
     plan.set_split(-1)
     got = run()
