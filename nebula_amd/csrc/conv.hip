@@ -149,7 +149,7 @@ enum { GATHER_PADDED = 0,   // any geometry: every tap is bounds-checked
 
 // OCC = blocks the register budget must leave room for on a CU (the persistent grid is sized with it)
 template<int MT, int NT, int WAVES_M, int WAVES_N, int OCC, int GATHER, bool FAST_ACT>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC)
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void conv_igemm_kernel(const ConvArgs a) {
     constexpr int BK = CONV_BK;
     constexpr int NTHREADS = 64 * WAVES_M * WAVES_N;
@@ -358,20 +358,24 @@ void conv_igemm_kernel(const ConvArgs a) {
     // pipe waits for, which is most of what a layer with few patch rows does.  The per-filter scale is
     // always applied (it is 1.0 where the layer has no batch normalisation, and acc * 1 + b rounds as
     // acc + b does).
-    auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff) {
-        constexpr bool SLOPED = decltype(sloped)::value, RES = decltype(with_residual)::value;
+    // (forced inline: called from four places, and as a real call it would take the accumulators through memory)
+    auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff, unsigned roff, int act, int post_act)
+                          __attribute__((always_inline)) {
+        // with_residual: 0 none, 1 at the output's own offsets (same shape), 2 at offsets of its own
+        constexpr bool SLOPED = decltype(sloped)::value, RES = decltype(with_residual)::value != 0,
+                       RES_OWN = decltype(with_residual)::value == 2;
         typedef float __attribute__((ext_vector_type(NT))) pixvec;
         const unsigned row_bytes = (unsigned)a.OHW * 4u;
         char *__restrict__ yb = reinterpret_cast<char*>(a.y);
         const char *__restrict__ rb = reinterpret_cast<const char*>(a.res);
-        const int act = a.act, post_act = a.post_act;
+        const unsigned res_row_bytes = (unsigned)a.res_hw * 4u;
         // per-filter constants one group of rows ahead of their use
-        float4 gv[2][MT], bv[2][MT];
+        vec4f gv[2][MT], bv[2][MT];
         auto load_constants = [&](int q) {
             #pragma unroll
             for(int u = 0; u < MT; u++) {
-                gv[q & 1][u] = *reinterpret_cast<const float4*>(a.g + f_lane + q * 8 * MT + 4 * u);
-                bv[q & 1][u] = *reinterpret_cast<const float4*>(a.b + f_lane + q * 8 * MT + 4 * u);
+                gv[q & 1][u] = *reinterpret_cast<const vec4f*>(a.g + f_lane + q * 8 * MT + 4 * u);
+                bv[q & 1][u] = *reinterpret_cast<const vec4f*>(a.b + f_lane + q * 8 * MT + 4 * u);
             }
         };
         load_constants(0);
@@ -382,7 +386,8 @@ void conv_igemm_kernel(const ConvArgs a) {
             if(RES) {
                 #pragma unroll
                 for(int e = 0; e < 4 * MT; e++)
-                    rv[e] = *reinterpret_cast<const pixvec*>(rb + (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes));
+                    rv[e] = *reinterpret_cast<const pixvec*>(rb + (RES_OWN ? (size_t)(roff + (unsigned)(q * 8 * MT + e) * res_row_bytes)
+                                                                           : (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes)));
             }
             #pragma unroll
             for(int e = 0; e < 4 * MT; e++) {
@@ -414,15 +419,41 @@ void conv_igemm_kernel(const ConvArgs a) {
         // 32-bit offset, so a row costs one integer add besides its arithmetic.  An instruction spent
         // here is an instruction the matrix pipe waits for, which is what layers with few patch rows
         // are made of.
-        if(a.short_epilogue && m0 + BM <= a.F && (NT == 1 || (a.OHW & 1) == 0)) {
+        // A fused shortcut with fewer channels than filters gives a tile's rows a residual either all or not at
+        // all (mixed tiles take the general path); a tile without one applies the two activations in a row, which
+        // is one activation when either is linear.  A strided or larger connection is read at its own row pitch;
+        // pairs of pixels (NT = 2) are one vector of it only at stride 1 and equal width.
+        const bool tile_res = a.res != NULL && m0 + BM <= a.res_c, tile_plain = a.res == NULL || m0 >= a.res_c;
+        if(a.short_epilogue && m0 + BM <= a.F && (NT == 1 || (a.OHW & 1) == 0) && (tile_res || tile_plain) &&
+           (!tile_res || NT == 1 || (a.res_stride == 1 && a.res_hw == a.OHW)) &&
+           (!tile_plain || a.res == NULL || a.act == NBL_ACT_LINEAR || a.post_act == NBL_ACT_LINEAR)) {
             const int f_lane = m0 + wm * MT * 32 + half * 4 * MT;
             const unsigned yoff = ((unsigned)(b0 * a.F + f_lane) * (unsigned)a.OHW + (unsigned)pix0) * 4u;
+            unsigned roff = 0;
+            int act = a.act, post_act = a.post_act;
+            if(tile_res) {
+                unsigned rpix = (unsigned)pix0;
+                if(a.res_hw != a.OHW || a.res_stride != 1) {
+                    const int h = pix0 / a.OW, w = pix0 - h * a.OW;
+                    rpix = (unsigned)(h * a.res_stride * a.res_w + w * a.res_stride);
+                }
+                roff = ((unsigned)(b0 * a.res_c + f_lane) * (unsigned)a.res_hw + rpix) * 4u;
+            } else if(a.res != NULL) {
+                act = a.act == NBL_ACT_LINEAR ? a.post_act : a.act;
+                post_act = NBL_ACT_LINEAR;
+            }
+            typedef std::integral_constant<int, 0> no_res;
+            typedef std::integral_constant<int, 1> res_at_output;
+            typedef std::integral_constant<int, 2> res_own;
+            const bool res_same_shape = a.res_c == a.F && a.res_hw == a.OHW && a.res_stride == 1;   // uniform
             if(a.short_epilogue == 1) {
-                if(a.res) short_epilogue(std::false_type(), std::true_type(), f_lane, yoff);
-                else short_epilogue(std::false_type(), std::false_type(), f_lane, yoff);
+                if(!tile_res) short_epilogue(std::false_type(), no_res(), f_lane, yoff, roff, act, post_act);
+                else if(res_same_shape) short_epilogue(std::false_type(), res_at_output(), f_lane, yoff, roff, act, post_act);
+                else short_epilogue(std::false_type(), res_own(), f_lane, yoff, roff, act, post_act);
             } else {
-                if(a.res) short_epilogue(std::true_type(), std::true_type(), f_lane, yoff);
-                else short_epilogue(std::true_type(), std::false_type(), f_lane, yoff);
+                if(!tile_res) short_epilogue(std::true_type(), no_res(), f_lane, yoff, roff, act, post_act);
+                else if(res_same_shape) short_epilogue(std::true_type(), res_at_output(), f_lane, yoff, roff, act, post_act);
+                else short_epilogue(std::true_type(), res_own(), f_lane, yoff, roff, act, post_act);
             }
             return;
         }
@@ -932,10 +963,13 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
                                 rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE);
     }
     const size_t out_bytes = (size_t)npix * p->F * sizeof(float);
-    const bool res_same_shape = rs && rs->c == p->F && rs->h == p->OH && rs->w == p->OW;
+    // the short epilogue reads a residual whose box covers the whole output plane (same size, or sub-sampled by the
+    // shortcut's stride) and that has no more channels than there are filters; residual tensor below 4 GiB
+    const bool res_plain_box = rs && rs->c <= p->F && a.res_box_h == (int)p->OH && a.res_box_w == (int)p->OW &&
+                               (size_t)B * rs->c * rs->h * rs->w * sizeof(float) < (1ull << 32);
     const bool sloped = p->act == NBL_ACT_LEAKY || p->act == NBL_ACT_RELIE ||
                         (rs && (rs->post_act == NBL_ACT_LEAKY || rs->post_act == NBL_ACT_RELIE));
-    a.short_epilogue = !(fast_act && out_bytes < (1ull << 32) && (!rs || res_same_shape) &&
+    a.short_epilogue = !(fast_act && out_bytes < (1ull << 32) && (!rs || res_plain_box) &&
                          ((size_t)y_dev & 7) == 0 && (!rs || ((size_t)rs->res & 7) == 0)) ? 0 : sloped ? 2 : 1;
     a.ttab = p->ttab_dev; a.ksize = (int)p->k; a.plane_bytes = p->H * p->W * 4u;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
