@@ -440,16 +440,18 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ part, float *__re
 // lanes 0-31 supply k+0..3 and lanes 32-63 k+4..7 of both operands (a legal pairing).  Loads run one
 // batch of U steps ahead; two accumulators take turns because with one wave per SIMD nothing else
 // hides the latency between two MFMAs on the same registers.  kw must be a multiple of 32.
+// astep / bstep: floats between a lane's pieces of consecutive 8-wide k blocks: 8 in a row-major matrix; 256 in the
+// operand-major layout below, where the 64 pieces one load instruction fetches are one contiguous KiB.
 __device__ __forceinline__ void wave_tile_from_global(const float *__restrict__ ap, const float *__restrict__ bp, int kw,
-                                                      floatx16 &acc0, floatx16 &acc1) {
+                                                      floatx16 &acc0, floatx16 &acc1, int astep = 8, int bstep = 8) {
     constexpr int U = 4;                    // 8-wide k steps per batch of loads
     const int nb = kw / (8 * U);
     float4 av[2][U], bv[2][U];
     auto load = [&](int buf, int b) {
         #pragma unroll
         for(int u = 0; u < U; u++) {
-            av[buf][u] = *reinterpret_cast<const float4*>(ap + (b * U + u) * 8);
-            bv[buf][u] = *reinterpret_cast<const float4*>(bp + (b * U + u) * 8);
+            av[buf][u] = *reinterpret_cast<const float4*>(ap + (size_t)(b * U + u) * astep);
+            bv[buf][u] = *reinterpret_cast<const float4*>(bp + (size_t)(b * U + u) * bstep);
         }
     };
     #pragma unroll
@@ -485,8 +487,20 @@ __device__ __forceinline__ void wave_tile_from_global(const float *__restrict__ 
 // unit): sum of the four partial tiles for each gate, bias, input-side pre-activation, the cell update
 // (lstm_layer.cc:264-312, each product rounded on its own) and h_t written into y[t], which is the
 // next step's operand.  Needs H % 128 == 0 and 16-byte aligned rows.
+// Operand-major layout of a [rows][K] matrix (rows and K padded to 32 and 8): the 16-byte piece lane (half, r) of
+// a wave feeds to the MFMAs of the 8-wide k block kb of row tile rt -- elements k = 8*kb + 4*half .. +3 of row
+// 32*rt + r -- sits at float offset ((rt * K/8 + kb) * 64 + half*32 + r) * 4.  A wave's load instruction then
+// reads one contiguous KiB (8 cache lines) where the row-major matrix makes it touch 32 lines for the same bytes;
+// with row-major operands the step kernels kept the CU's address unit busy for 6 of their 9 us.
+__host__ __device__ inline size_t opmajor_offset(unsigned row, unsigned k, unsigned K) {
+    return (((size_t)(row / 32) * (K / 8) + k / 8) * 64 + ((k % 8) / 4) * 32 + row % 32) * 4 + k % 4;
+}
+
 struct LstmStepArgs {
-    const float *hprev; const float *w; const float *gx; const float *bw; float *c; float *hout;
+    const float *hprev_op;      // h_{t-1}, operand-major [ceil(B/32)*32][H]
+    const float *w_op;          // recurrent weights, operand-major [Np][H]
+    const float *gx; const float *bw; float *c; float *hout;
+    float *hnext_op;            // h_t in operand-major layout for the next step
     int B, H, Np, sub_act;
 };
 
@@ -497,10 +511,9 @@ void lstm_step_kernel(const LstmStepArgs a) {
     const int r = lane & 31, half = lane >> 5;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int kw = a.H >> 2;                // k range of one wave
-    const int arow = min(m0 + r, a.B - 1);  // rows past the batch repeat the last one; their sums are dropped
-    floatx16 acc0, acc1;
-    wave_tile_from_global(a.hprev + (size_t)arow * a.H + wave * kw + half * 4,
-                          a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4, kw, acc0, acc1);
+    floatx16 acc0, acc1;                    // (rows past the batch hold zeros in the operand-major h; their sums are dropped)
+    wave_tile_from_global(a.hprev_op + opmajor_offset(m0 + r, wave * kw + half * 4, a.H),
+                          a.w_op + opmajor_offset(n0 + r, wave * kw + half * 4, a.H), kw, acc0, acc1, 256, 256);
 
     // accumulator register i of a 32x32 tile: row 8*(i/4) + 4*(lane/32) + i%4 (batch), column lane%32 (gate column)
     #pragma unroll
@@ -525,15 +538,21 @@ void lstm_step_kernel(const LstmStepArgs a) {
     const float cf = __fmul_rn(a.c[e], gf);
     const float ct = __fadd_rn(cf, ig);
     a.c[e] = ct;
-    a.hout[e] = __fmul_rn(lstm_tanh(ct), go);
+    const float ht = __fmul_rn(lstm_tanh(ct), go);
+    a.hout[e] = ht;
+    a.hnext_op[opmajor_offset(m, h, a.H)] = ht;
 }
 
 // One step of the RNN layer's recurrence (rnn_layer.cc:100-115) in one launch, same work split as
 // lstm_step_kernel: hid = act((prev . Wh^T) * g + b), state = in_t + hid; a block owns a 32x32 tile of
 // the [B x O] step.  hid is also stored where the caller wants it (step 0's output gate reads it).
 struct RnnStepArgs {
-    const float *prev; const float *w; const float *g; const float *b; const float *in_t;
+    const float *prev;               // row-major [B][H] (step 0: the input gate's output) or operand-major
+    int prev_opmajor;
+    const float *w_op;               // hidden gate's weights, operand-major [H][H]
+    const float *g; const float *b; const float *in_t;
     float *state; float *hid;        // hid may be NULL
+    float *state_op;                 // the new state once more, operand-major, for the next step
     int B, H, act;                   // H = layer width (rows of Wh and its fan-in)
 };
 
@@ -544,10 +563,12 @@ void rnn_step_kernel(const RnnStepArgs a) {
     const int r = lane & 31, half = lane >> 5;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int kw = a.H >> 2;
-    const int arow = min(m0 + r, a.B - 1);
+    const int arow = min(m0 + r, a.B - 1);  // row-major operand: rows past the batch repeat the last one; their sums are dropped
     floatx16 acc0, acc1;
-    wave_tile_from_global(a.prev + (size_t)arow * a.H + wave * kw + half * 4,
-                          a.w + (size_t)(n0 + r) * a.H + wave * kw + half * 4, kw, acc0, acc1);
+    wave_tile_from_global(a.prev_opmajor ? a.prev + opmajor_offset(m0 + r, wave * kw + half * 4, a.H)
+                                         : a.prev + (size_t)arow * a.H + wave * kw + half * 4,
+                          a.w_op + opmajor_offset(n0 + r, wave * kw + half * 4, a.H), kw, acc0, acc1,
+                          a.prev_opmajor ? 256 : 8, 256);
     #pragma unroll
     for(int i = 0; i < 16; i++) red[wave][8 * (i >> 2) + 4 * half + (i & 3)][r] = acc0[i] + acc1[i];
     __syncthreads();
@@ -565,8 +586,9 @@ void rnn_step_kernel(const RnnStepArgs a) {
     const size_t e = (size_t)m * a.H + n0 + c4;
     const float4 in = *reinterpret_cast<const float4*>(a.in_t + e);
     if(a.hid) *reinterpret_cast<float4*>(a.hid + e) = make_float4(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<float4*>(a.state + e) = make_float4(__fadd_rn(in.x, v[0]), __fadd_rn(in.y, v[1]),
-                                                          __fadd_rn(in.z, v[2]), __fadd_rn(in.w, v[3]));
+    const float4 st = make_float4(__fadd_rn(in.x, v[0]), __fadd_rn(in.y, v[1]), __fadd_rn(in.z, v[2]), __fadd_rn(in.w, v[3]));
+    *reinterpret_cast<float4*>(a.state + e) = st;
+    *reinterpret_cast<float4*>(a.state_op + opmajor_offset(m, n0 + c4, a.H)) = st;     // four adjacent k: one piece
 }
 
 // state = a + b elementwise (the two axpy of rnn_layer.cc:108-115 on a zeroed state)
@@ -658,6 +680,8 @@ struct nbl_lstm_plan {
     int sub_act;
     float *ucat_dev;                    // [4*Hp][I]  input-side weights, interleaved gate order, BN scale folded in
     float *wcat_dev;                    // [4*Hp][H]  recurrent-side weights, same order
+    float *wcat_op_dev;                 // the same matrix in operand-major layout (gate interleave 8 only)
+    float *hop_dev[2]; size_t hop_bytes; // h_{t-1} / h_t in operand-major layout, [ceil(B/32)*32][H] each
     float *bu_dev, *bw_dev;             // [4*Hp] biases (BN shift folded in); for a linear sub_act bw is folded into bu
     float *gx_dev; float *h0_dev; float *c_dev; size_t gx_bytes, state_bytes;
     float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
@@ -670,6 +694,8 @@ struct nbl_rnn_plan {
     unsigned I, O;
     nbl_fc_plan *gate[3];
     float *in_all, *states, *hid0, *tmp;     // [T*B][O], [T*B][O], [B][O], [B][O]
+    float *wh_op;                            // hidden gate's weights in operand-major layout (O % 128 == 0)
+    float *sop[2]; size_t sop_bytes;         // state of the previous / this step in operand-major layout
     size_t rows_alloc, seqs_alloc;
 };
 
@@ -855,6 +881,16 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
     if(sub_act == NBL_ACT_LINEAR)
         for(unsigned n = 0; n < Np; n++) { bu[n] = bu[n] + bw[n]; bw[n] = 0.0f; }
     int rc;
+    if(p->G == 8) {        // the per-step kernel reads the recurrent weights in operand-major order (H % 128 == 0 here)
+        std::vector<float> wop((size_t)Np * H);
+        for(unsigned n = 0; n < Np; n++)
+            for(unsigned k = 0; k < H; k++) wop[opmajor_offset(n, k, H)] = wcat[(size_t)n * H + k];
+        if((rc = nbl_malloc(ctx, (void**)&p->wcat_op_dev, wop.size() * sizeof(float))) != NBL_OK ||
+           (rc = nbl_h2d(ctx, p->wcat_op_dev, wop.data(), wop.size() * sizeof(float))) != NBL_OK) {
+            nbl_lstm_plan_destroy(ctx, p);
+            return rc;
+        }
+    }
     if((rc = nbl_malloc(ctx, (void**)&p->ucat_dev, ucat.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->wcat_dev, wcat.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->bu_dev, Np * sizeof(float))) != NBL_OK ||
@@ -874,7 +910,7 @@ int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->ucat_dev); nbl_free(ctx, p->wcat_dev); nbl_free(ctx, p->bu_dev); nbl_free(ctx, p->bw_dev);
     nbl_free(ctx, p->gx_dev); nbl_free(ctx, p->h0_dev); nbl_free(ctx, p->c_dev); nbl_free(ctx, p->part_dev);
-    nbl_free(ctx, p->ucat_t_dev);
+    nbl_free(ctx, p->ucat_t_dev); nbl_free(ctx, p->wcat_op_dev); nbl_free(ctx, p->hop_dev[0]); nbl_free(ctx, p->hop_dev[1]);
     delete p;
     return NBL_OK;
 }
@@ -904,6 +940,19 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
     // zero initial hidden and cell state (first forward() of a fresh reference layer)
     if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK)
         return rc;
+    const size_t hop_need = (size_t)nbl_div_up(B, 32) * 32 * p->H * sizeof(float);
+    if(p->G == 8) {
+        if(p->hop_bytes < hop_need) {
+            if((rc = nbl_free(ctx, p->hop_dev[0])) != NBL_OK || (rc = nbl_free(ctx, p->hop_dev[1])) != NBL_OK) return rc;
+            p->hop_dev[0] = p->hop_dev[1] = NULL; p->hop_bytes = 0;
+            if((rc = nbl_malloc(ctx, (void**)&p->hop_dev[0], hop_need)) != NBL_OK ||
+               (rc = nbl_malloc(ctx, (void**)&p->hop_dev[1], hop_need)) != NBL_OK) return rc;
+            p->hop_bytes = hop_need;
+        }
+        // h_{-1} = 0, and rows past the batch stay zero in both buffers (the step kernel writes real rows only)
+        if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->hop_dev[1], hop_need)) != NBL_OK)
+            return rc;
+    }
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
     if(tokens_dev) {
         if(!p->ucat_t_dev) {
@@ -920,14 +969,13 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
     const size_t step = (size_t)B * p->H;
     if(p->G == 8) {
         // Recurrent half, one launch per step (lstm_step_kernel).  h_{t-1} is read straight from y[t-1].
-        if(!aligned16(y_dev) || !aligned16(p->wcat_dev) || !aligned16(p->h0_dev))
-            return nbl_fail(ctx, NBL_EINVAL, "nbl_lstm_fwd: y_dev must be 16-byte aligned");
         LstmStepArgs sa;
-        sa.w = p->wcat_dev; sa.bw = p->bw_dev; sa.c = p->c_dev; sa.B = (int)B; sa.H = (int)p->H; sa.Np = (int)Np;
+        sa.w_op = p->wcat_op_dev; sa.bw = p->bw_dev; sa.c = p->c_dev; sa.B = (int)B; sa.H = (int)p->H; sa.Np = (int)Np;
         sa.sub_act = p->sub_act;
         const dim3 grid(Np / 32, nbl_div_up(B, 32));
         for(unsigned t = 0; t < T; t++) {
-            sa.hprev = t == 0 ? p->h0_dev : y_dev + (size_t)(t - 1) * step;
+            sa.hprev_op = p->hop_dev[t & 1];
+            sa.hnext_op = p->hop_dev[(t + 1) & 1];
             sa.gx = p->gx_dev + (size_t)t * B * Np;
             sa.hout = y_dev + (size_t)t * step;
             hipLaunchKernelGGL(lstm_step_kernel, grid, dim3(256), 0, ctx->stream, sa);
@@ -1015,6 +1063,17 @@ int nbl_rnn_pack(nbl_ctx *ctx, const float *const *weight_host, const float *con
                                    s == 0 ? I : O, O, act, &p->gate[s]);
         if(rc != NBL_OK) { nbl_rnn_plan_destroy(ctx, p); return rc; }
     }
+    if(O % 128 == 0) {      // the per-step kernel reads the hidden gate's weights in operand-major order
+        std::vector<float> wop((size_t)O * O);
+        for(unsigned n = 0; n < O; n++)
+            for(unsigned k = 0; k < O; k++) wop[opmajor_offset(n, k, O)] = weight_host[1][(size_t)n * O + k];
+        int rc;
+        if((rc = nbl_malloc(ctx, (void**)&p->wh_op, wop.size() * sizeof(float))) != NBL_OK ||
+           (rc = nbl_h2d(ctx, p->wh_op, wop.data(), wop.size() * sizeof(float))) != NBL_OK) {
+            nbl_rnn_plan_destroy(ctx, p);
+            return rc;
+        }
+    }
     *out = p;
     return NBL_OK;
 }
@@ -1023,6 +1082,7 @@ int nbl_rnn_plan_destroy(nbl_ctx *ctx, nbl_rnn_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     for(int s = 0; s < 3; s++) if(p->gate[s]) nbl_fc_plan_destroy(ctx, p->gate[s]);
     nbl_free(ctx, p->in_all); nbl_free(ctx, p->states); nbl_free(ctx, p->hid0); nbl_free(ctx, p->tmp);
+    nbl_free(ctx, p->wh_op); nbl_free(ctx, p->sop[0]); nbl_free(ctx, p->sop[1]);
     delete p;
     return NBL_OK;
 }
@@ -1050,8 +1110,21 @@ int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev,
     if((rc = launch_fc(ctx, x_dev, gi->w_dev, p->in_all, (int)rows, (int)p->O, (int)p->I, gi->g_dev, gi->b_dev,
                        gi->act, gi->has_scale, &gi->ws_dev, &gi->ws_bytes)) != NBL_OK) return rc;
     const size_t step = (size_t)B * p->O;
-    const bool one_launch = p->O % 128 == 0 && aligned16(gh->w_dev) && aligned16(p->in_all) && aligned16(p->states) &&
-                            aligned16(p->hid0);
+    const bool one_launch = p->wh_op != NULL && aligned16(p->in_all) && aligned16(p->states) && aligned16(p->hid0);
+    if(one_launch) {
+        const size_t need = (size_t)nbl_div_up(B, 32) * 32 * p->O * sizeof(float);
+        if(p->sop_bytes < need) {
+            if((rc = nbl_free(ctx, p->sop[0])) != NBL_OK || (rc = nbl_free(ctx, p->sop[1])) != NBL_OK) return rc;
+            p->sop[0] = p->sop[1] = NULL; p->sop_bytes = 0;
+            if((rc = nbl_malloc(ctx, (void**)&p->sop[0], need)) != NBL_OK ||
+               (rc = nbl_malloc(ctx, (void**)&p->sop[1], need)) != NBL_OK) return rc;
+            p->sop_bytes = need;
+            // rows past the batch are read (their sums are dropped) and must hold numbers: zero once, the kernel
+            // writes real rows only
+            if((rc = nbl_fill_zero(ctx, p->sop[0], need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->sop[1], need)) != NBL_OK)
+                return rc;
+        }
+    }
     for(unsigned t = 0; t < T; t++) {
         // rnn_layer.cc:103-104: step 0's hidden gate reads the input gate's output, later steps the previous state
         const float *prev = t == 0 ? p->in_all : p->states + (size_t)(t - 1) * step;
@@ -1059,7 +1132,9 @@ int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev,
         float *state = p->states + (size_t)t * step;
         if(one_launch) {
             RnnStepArgs a;
-            a.prev = prev; a.w = gh->w_dev; a.g = gh->g_dev; a.b = gh->b_dev; a.in_t = in_t; a.state = state;
+            a.prev = t == 0 ? prev : p->sop[(t - 1) & 1]; a.prev_opmajor = t == 0 ? 0 : 1;
+            a.w_op = p->wh_op; a.state_op = p->sop[t & 1];
+            a.g = gh->g_dev; a.b = gh->b_dev; a.in_t = in_t; a.state = state;
             a.hid = t == 0 ? p->hid0 : NULL; a.B = (int)B; a.H = (int)p->O; a.act = gh->act;
             hipLaunchKernelGGL(rnn_step_kernel, dim3(p->O / 32, nbl_div_up(B, 32)), dim3(256), 0, ctx->stream, a);
             NBL_LAUNCH_CHECK(ctx, "rnn_step_kernel");
