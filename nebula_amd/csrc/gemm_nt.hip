@@ -511,6 +511,18 @@ void lstm_step_kernel(const LstmStepArgs a) {
     const int r = lane & 31, half = lane >> 5;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int kw = a.H >> 2;                // k range of one wave
+    // what the cell update needs besides the products is requested first and arrives behind the k loop
+    const int ml = tid >> 3, hh = tid & 7;
+    const int m = m0 + ml, h = blockIdx.x * 8 + hh;
+    const bool live = m < a.B;
+    const size_t e = (size_t)(live ? m : 0) * a.H + h;
+    float gxv[4], bwv[4];
+    #pragma unroll
+    for(int gate = 0; gate < 4; gate++) {
+        gxv[gate] = a.gx[(size_t)(live ? m : 0) * a.Np + n0 + gate * 8 + hh];
+        bwv[gate] = a.bw[n0 + gate * 8 + hh];
+    }
+    const float cprev = a.c[e];
     floatx16 acc0, acc1;                    // (rows past the batch hold zeros in the operand-major h; their sums are dropped)
     wave_tile_from_global(a.hprev_op + opmajor_offset(m0 + r, wave * kw + half * 4, a.H),
                           a.w_op + opmajor_offset(n0 + r, wave * kw + half * 4, a.H), kw, acc0, acc1, 256, 256);
@@ -519,23 +531,20 @@ void lstm_step_kernel(const LstmStepArgs a) {
     #pragma unroll
     for(int i = 0; i < 16; i++) red[wave][8 * (i >> 2) + 4 * half + (i & 3)][r] = acc0[i] + acc1[i];
     __syncthreads();
-    const int ml = tid >> 3, hh = tid & 7;
-    const int m = m0 + ml, h = blockIdx.x * 8 + hh;
-    if(m >= a.B) return;
+    if(!live) return;
     float pre[4];
     #pragma unroll
     for(int gate = 0; gate < 4; gate++) {
         const int col = gate * 8 + hh;
-        const float t = ((red[0][ml][col] + red[1][ml][col]) + (red[2][ml][col] + red[3][ml][col])) + a.bw[n0 + col];
-        pre[gate] = (a.sub_act == NBL_ACT_LINEAR ? t : nbl_act_apply(a.sub_act, t)) + a.gx[(size_t)m * a.Np + n0 + col];
+        const float t = ((red[0][ml][col] + red[1][ml][col]) + (red[2][ml][col] + red[3][ml][col])) + bwv[gate];
+        pre[gate] = (a.sub_act == NBL_ACT_LINEAR ? t : nbl_act_apply(a.sub_act, t)) + gxv[gate];
     }
     const float gi = lstm_logistic(pre[0]);
     const float gf = lstm_logistic(pre[1]);
     const float gg = lstm_tanh(pre[2]);
     const float go = lstm_logistic(pre[3]);
-    const size_t e = (size_t)m * a.H + h;
     const float ig = __fmul_rn(gi, gg);
-    const float cf = __fmul_rn(a.c[e], gf);
+    const float cf = __fmul_rn(cprev, gf);
     const float ct = __fadd_rn(cf, ig);
     a.c[e] = ct;
     const float ht = __fmul_rn(lstm_tanh(ct), go);
@@ -564,6 +573,13 @@ void rnn_step_kernel(const RnnStepArgs a) {
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int kw = a.H >> 2;
     const int arow = min(m0 + r, a.B - 1);  // row-major operand: rows past the batch repeat the last one; their sums are dropped
+    // what follows the products is requested first and arrives behind the k loop
+    const int ml = tid >> 3, c4 = (tid & 7) * 4;
+    const int m = m0 + ml;
+    const bool live = m < a.B;
+    const size_t e = (size_t)(live ? m : 0) * a.H + n0 + c4;
+    const float4 in = *reinterpret_cast<const float4*>(a.in_t + e);
+    const float4 gq = *reinterpret_cast<const float4*>(a.g + n0 + c4), bq = *reinterpret_cast<const float4*>(a.b + n0 + c4);
     floatx16 acc0, acc1;
     wave_tile_from_global(a.prev_opmajor ? a.prev + opmajor_offset(m0 + r, wave * kw + half * 4, a.H)
                                          : a.prev + (size_t)arow * a.H + wave * kw + half * 4,
@@ -573,18 +589,15 @@ void rnn_step_kernel(const RnnStepArgs a) {
     for(int i = 0; i < 16; i++) red[wave][8 * (i >> 2) + 4 * half + (i & 3)][r] = acc0[i] + acc1[i];
     __syncthreads();
     // thread -> 4 adjacent columns of one row
-    const int ml = tid >> 3, c4 = (tid & 7) * 4;
-    const int m = m0 + ml;
-    if(m >= a.B) return;
+    if(!live) return;
+    const float gs[4] = { gq.x, gq.y, gq.z, gq.w }, bs[4] = { bq.x, bq.y, bq.z, bq.w };
     float v[4];
     #pragma unroll
     for(int j = 0; j < 4; j++) {
-        const int col = c4 + j, n = n0 + col;
+        const int col = c4 + j;
         const float sum = (red[0][ml][col] + red[1][ml][col]) + (red[2][ml][col] + red[3][ml][col]);
-        v[j] = nbl_act_apply(a.act, __builtin_fmaf(sum, a.g[n], a.b[n]));
+        v[j] = nbl_act_apply(a.act, __builtin_fmaf(sum, gs[j], bs[j]));
     }
-    const size_t e = (size_t)m * a.H + n0 + c4;
-    const float4 in = *reinterpret_cast<const float4*>(a.in_t + e);
     if(a.hid) *reinterpret_cast<float4*>(a.hid + e) = make_float4(v[0], v[1], v[2], v[3]);
     const float4 st = make_float4(__fadd_rn(in.x, v[0]), __fadd_rn(in.y, v[1]), __fadd_rn(in.z, v[2]), __fadd_rn(in.w, v[3]));
     *reinterpret_cast<float4*>(a.state + e) = st;
