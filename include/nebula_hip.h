@@ -135,7 +135,9 @@ int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigne
  * arrays in .wgh order bias[O], weight[O][I], [scale, mean, var][O] or NULLs.
  * nbl_fc_fwd: connected_layer_t::_forward_() (models/layers/connected_layer.cu:19-53; CPU twin
  * connected_layer.cc:245-277): y[B][O] = act((x[B][I] . W^T) * g + b).  (The CUDA file adds bias[0]
- * to every output, connected_layer.cu:44; the CPU file is followed.) */
+ * to every output, connected_layer.cu:44; the CPU file is followed.)  A plan whose fan-in is a multiple
+ * of 32 holds its weights twice on the device: row-major, and as contiguous 16 KB tiles for the streaming
+ * kernel. */
 int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
                 const float *scale_host, const float *mean_host, const float *var_host,
                 unsigned I, unsigned O, int act, nbl_fc_plan **out);
