@@ -1011,8 +1011,7 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
         p->state_bytes = st_need;
     }
     // zero initial hidden and cell state (first forward() of a fresh reference layer)
-    if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK)
-        return rc;
+    if((rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK) return rc;
     const size_t hop_need = (size_t)nbl_div_up(B, 32) * 32 * p->H * sizeof(float);
     if(p->G == 8) {
         if(p->hop_bytes < hop_need) {
@@ -1021,11 +1020,12 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
             if((rc = nbl_malloc(ctx, (void**)&p->hop_dev[0], hop_need)) != NBL_OK ||
                (rc = nbl_malloc(ctx, (void**)&p->hop_dev[1], hop_need)) != NBL_OK) return rc;
             p->hop_bytes = hop_need;
+            // rows past the batch are read (their sums are dropped) and must hold numbers; the step kernel writes
+            // real rows only, so zeroing once is enough for the buffer step 0 writes
+            if((rc = nbl_fill_zero(ctx, p->hop_dev[1], hop_need)) != NBL_OK) return rc;
         }
-        // h_{-1} = 0, and rows past the batch stay zero in both buffers (the step kernel writes real rows only)
-        if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK || (rc = nbl_fill_zero(ctx, p->hop_dev[1], hop_need)) != NBL_OK)
-            return rc;
-    }
+        if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK) return rc;      // h_{-1} = 0
+    } else if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK) return rc;
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
     if(tokens_dev) {
         if(!p->ucat_t_dev) {
