@@ -481,5 +481,8 @@ def test_error_paths(ctx):
     # zero batch is a no-op, not an error
     plan = ctx.conv_pack(w, b, None, H=8, W=8, stride=1, pad=1, act="relu")
     assert l.nbl_conv2d_fwd(ctx.h, plan.p, d.ptr, d.ptr, 0) == 0
+    # k-split modes: -1 (measured), 0, 1 and a slice count of 2..8
+    assert l.nbl_conv2d_plan_set_split(plan.p, 9) != 0 and l.nbl_conv2d_plan_set_split(plan.p, -2) != 0
+    assert l.nbl_conv2d_plan_set_split(plan.p, 8) == 0 and l.nbl_conv2d_plan_set_split(plan.p, -1) == 0
     assert l.nbl_ctx_create(99, C.byref(p)) != 0
     assert b"device" in l.nbl_last_error(None)
