@@ -126,6 +126,41 @@ void pool_pair_kernel(const float *__restrict__ x, float *__restrict__ y, unsign
     if(IS_MAX && WRITE_INDEX) *reinterpret_cast<uint2*>(index + o) = make_uint2(at[0], at[1]);
 }
 
+// Average over whole planes (window = plane, stride = window, no padding: the pool that ends ResNet).  The
+// planes are contiguous, so a block stages AVG_PLANES consecutive planes through LDS with 16-byte loads and
+// then one thread per plane adds its plane's floats in scan order (the order of pooling_layer.cc:161-170).
+// LDS rows have an odd stride so that the threads of a wave read different banks.
+constexpr int AVG_PLANES = 128;
+__global__ __launch_bounds__(256)
+void avgpool_plane_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned planes, unsigned hw, float divisor) {
+    extern __shared__ float staged[];
+    const unsigned row = hw | 1u;
+    const unsigned first = blockIdx.x * AVG_PLANES;
+    const unsigned here = min((unsigned)AVG_PLANES, planes - first);
+    const unsigned count = here * hw;
+    const float *__restrict__ src = x + (size_t)first * hw;
+    for(unsigned v = threadIdx.x; v < count / 4; v += 256) {
+        const float4 q = *reinterpret_cast<const float4*>(src + 4 * v);
+        const float e[4] = { q.x, q.y, q.z, q.w };
+        #pragma unroll
+        for(unsigned c = 0; c < 4; c++) {
+            const unsigned i = 4 * v + c, p = i / hw;
+            staged[p * row + (i - p * hw)] = e[c];
+        }
+    }
+    for(unsigned i = (count & ~3u) + threadIdx.x; i < count; i += 256) {
+        const unsigned p = i / hw;
+        staged[p * row + (i - p * hw)] = src[i];
+    }
+    __syncthreads();
+    if(threadIdx.x < here) {
+        const float *mine = staged + threadIdx.x * row;
+        float acc = 0.0f;
+        for(unsigned e = 0; e < hw; e++) acc += mine[e];
+        y[first + threadIdx.x] = acc / divisor;
+    }
+}
+
 // ---- shortcut ------------------------------------------------------------------------------------
 // y = act(prev + conn') where conn' is conn cropped to the common channel/height/width box and
 // sampled with stride = max(1, in_w/out_w), sample = max(1, out_w/in_w) (common/utils.cc:28-60).
@@ -423,6 +458,15 @@ int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index
         }
 #undef NBL_PAIR_LAUNCH
         NBL_LAUNCH_CHECK(ctx, "pool_pair_kernel");
+        return NBL_OK;
+    }
+    // the window is the whole plane: contiguous planes staged through LDS
+    if(mode == NBL_POOL_AVG && pad == 0 && ksize == H && ksize == W && OH == 1 && OW == 1 &&
+       (size_t)AVG_PLANES * ((H * W) | 1u) * sizeof(float) <= 64 * 1024 && ((size_t)x_dev & 15) == 0) {
+        const unsigned planes = B * C, hw = H * W;
+        hipLaunchKernelGGL(avgpool_plane_kernel, dim3(nbl_div_up(planes, (unsigned)AVG_PLANES)), dim3(256),
+                           AVG_PLANES * (hw | 1u) * sizeof(float), ctx->stream, x_dev, y_dev, planes, hw, (float)(ksize * ksize));
+        NBL_LAUNCH_CHECK(ctx, "avgpool_plane_kernel");
         return NBL_OK;
     }
     dim3 grid((unsigned)nbl_div_up_sz(total, 256)), block(256);

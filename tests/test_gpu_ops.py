@@ -270,6 +270,27 @@ def test_avgpool_bit_exact(ctx, geom):
     np.testing.assert_array_equal(bits(got), bits(want))
 
 
+# window = whole plane (the pool that ends ResNet): more planes than one block stages, even and odd plane
+# sizes, a plane count that leaves a ragged last block, a stride shorter than the window, and a plane too
+# large for the staged kernel (general kernel)
+PLANE_AVG = [(2, 130, 4, 4, 4, 4, 0), (1, 1, 3, 3, 3, 3, 0), (2, 3, 11, 11, 11, 11, 0), (1, 300, 7, 7, 7, 5, 0),
+             (1, 2, 12, 12, 12, 12, 0), (4, 512, 7, 7, 7, 7, 0)]
+
+
+@pytest.mark.parametrize("geom", PLANE_AVG)
+def test_avgpool_whole_plane_bit_exact(ctx, geom):
+    announce("avgpool whole plane", geom)
+    B, Cc, H, W, k, s, p = geom
+    rng = np.random.default_rng(sum(geom) + 2)
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    got = ctx.pool(ctx.array(x), k, s, p, "avg").numpy()
+    want = ob.avgpool_forward(x, k, s, p)
+    assert got.shape == (B, Cc, 1, 1)
+    np.testing.assert_array_equal(bits(got), bits(want))
+    # closed form: the mean of the plane
+    np.testing.assert_allclose(got[:, :, 0, 0], x.reshape(B, Cc, -1).astype(np.float64).mean(axis=2), rtol=0, atol=2e-6)
+
+
 SHORTCUT = [((2, 4, 9, 9), (2, 16, 9, 9)), ((2, 8, 10, 10), (2, 16, 5, 5)), ((1, 6, 19, 19), (1, 6, 10, 10)),
             ((2, 8, 4, 4), (2, 4, 8, 8)), ((3, 5, 7, 7), (3, 5, 7, 7)), ((2, 16, 8, 8), (2, 16, 8, 8)),
             ((2, 8, 12, 12), (2, 32, 12, 12)), ((2, 32, 12, 12), (2, 8, 12, 12)), ((2, 8, 7, 7), (2, 8, 7, 7)),
