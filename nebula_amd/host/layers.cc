@@ -29,7 +29,7 @@ layer_t::layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_lay
     layer_type(m_layer_type), activation_type(UNDEFINED_ACTIVATION),
     input_height(1), input_width(1), input_channel(1), input_size(1),
     output_height(1), output_width(1), output_channel(1), output_size(0),
-    output_data(NULL), delta(NULL), output_data_pinned(false),
+    output_data(NULL), output_data_pinned(false), delta(NULL),
     padding(0), num_filters(1), filter_size(1), stride(1), group(1),
     prev_layer(m_prev_layer), next_layer(NULL),
     output_data_dev(NULL), delta_dev(NULL),

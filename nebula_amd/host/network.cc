@@ -66,8 +66,9 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    last_step_only(false), fuse_shortcut(false), first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false),
-    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), image_staging_dev(NULL), image_staging_bytes(0), tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL) {
+    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), last_step_only(false), fuse_shortcut(false),
+    first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false), image_staging_dev(NULL),
+    tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL), image_staging_bytes(0) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
