@@ -239,6 +239,8 @@ def main():
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--graph", type=int, default=0, help="1: forward passes are replays of a recorded HIP graph, 0 (default): eager "
+                    "launches (the passes are GPU-bound on this machine: both take the same time)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every layer is batch-parallel with no exchange; "
@@ -269,6 +271,10 @@ def main():
     n_in = net.batch_size * net.input_size
     x = (rng.random(n_in, dtype=np.float32) if xdist == "uniform" else rng.standard_normal(n_in).astype(np.float32))
     net.set_input(x)                     # resident in HBM before the timed region
+    use_graph = args.graph == 1
+    if use_graph:
+        net.set_graph(True)              # pass 1 eager, pass 2 recorded, replays from pass 3 (all inside the warm-up)
+        args.warmup = max(args.warmup, 3)
 
     for _ in range(args.warmup):
         net.forward()
@@ -348,7 +354,8 @@ def main():
         "value": round(value, 2), "unit": "sequences/s" if is_lstm else "images/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded"},
+        "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded",
+                   "launch": "hip graph replay" if use_graph and net.graph_active else "eager"},
         "roofline": roofline,
     }
 

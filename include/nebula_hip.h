@@ -68,6 +68,10 @@ int nbl_malloc_host(nbl_ctx *ctx, void **host_ptr, size_t bytes);
 int nbl_free_host(nbl_ctx *ctx, void *host_ptr);
 int nbl_h2d(nbl_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);   /* returns after the copy */
 int nbl_d2h(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);   /* returns after the copy */
+/* The same copy queued on the context's stream without waiting for it (dst_host should be page-locked, from
+ * nbl_malloc_host; the data is there after the next nbl_sync).  This is the form a stream capture can record: the
+ * reference's blocking cudaMemcpy of the softmax output (models/layers/softmax_layer.cu:38-39) becomes a copy node. */
+int nbl_d2h_async(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
 int nbl_fill_zero(nbl_ctx *ctx, void *dst_dev, size_t bytes);                   /* a fill kernel, capturable */
 /* Device-to-device copy as a kernel on the context's stream (capturable; ranges must not overlap; both
  * pointers 16-byte aligned).  Replaces the reference's cudaMemcpy(..., cudaMemcpyDeviceToDevice) between

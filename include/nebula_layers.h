@@ -74,6 +74,16 @@ int nbl_net_layer_output(nbl_net *net, int layer, float *host, size_t count);
 int nbl_net_pool_index(nbl_net *net, int layer, unsigned *host, size_t count);
 /* the softmax layer skips its device->host copy when enabled = 0 (throughput measurement) */
 int nbl_net_softmax_copy(nbl_net *net, int enabled);
+/* enabled = 1 (also the [net] key hip_graph=1, which the reference ignores): nbl_net_forward records the
+ * launches of one pass into a HIP graph and replays it from then on: one launch on the host per pass instead
+ * of one per kernel (a recurrent net launches a kernel per layer and time step).  The first pass of a
+ * configuration runs eagerly (tile search, workspace growth), the second is recorded, later ones replay; a
+ * pass then always ends with a wait for the stream.  Loading weights, switching between token and dense
+ * input or toggling the softmax copy starts over.  The reference has no counterpart (its launches are eager).
+ * nbl_net_graph_active: 1 while passes are replays of a recorded graph, 0 otherwise (also when recording was
+ * not possible and the network stayed eager). */
+int nbl_net_set_graph(nbl_net *net, int enabled);
+int nbl_net_graph_active(nbl_net *net);
 /* the nbl_ctx* of the network (include/nebula_hip.h), e.g. for nbl_timer_start/stop */
 void *nbl_net_ctx(nbl_net *net);
 

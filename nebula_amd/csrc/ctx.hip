@@ -150,6 +150,14 @@ int nbl_d2h(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
     return NBL_OK;
 }
 
+int nbl_d2h_async(nbl_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    if(!ctx) return NBL_EINVAL;
+    if(bytes == 0) return NBL_OK;
+    NBL_REQUIRE(ctx, dst_host && src_dev, "nbl_d2h_async: NULL pointer");
+    NBL_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    return NBL_OK;
+}
+
 __global__ void nbl_fill_zero_kernel(uint4 *dst4, size_t n4, unsigned char *tail, unsigned ntail) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;

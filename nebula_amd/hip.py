@@ -32,6 +32,7 @@ SIGNATURES = {
     "nbl_free": (C.c_int, [_vp, _vp]),
     "nbl_h2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_d2h": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
+    "nbl_d2h_async": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_malloc_host": (C.c_int, [_vp, C.POINTER(_vp), C.c_size_t]),
     "nbl_free_host": (C.c_int, [_vp, _vp]),
     "nbl_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),

@@ -65,7 +65,7 @@ int nbl_net_destroy(nbl_net *n) {
 }
 
 int nbl_net_load_weights(nbl_net *n, const char *weight_path) {
-    NBL_NET_TRY(if(!n || !weight_path) throw std::runtime_error("NULL argument"); n->net->init_weight(weight_path));
+    NBL_NET_TRY(if(!n || !weight_path) throw std::runtime_error("NULL argument"); n->net->invalidate_graph(); n->net->init_weight(weight_path));
 }
 
 int nbl_net_store_weights(nbl_net *n, const char *weight_path) {
@@ -179,6 +179,15 @@ int nbl_net_softmax_copy(nbl_net *n, int enabled) {
             static_cast<softmax_layer_t*>(n->net->layers[i])->copy_to_host = enabled != 0;
     return 0;
 }
+
+int nbl_net_set_graph(nbl_net *n, int enabled) {
+    if(!n) return -1;
+    n->net->invalidate_graph();
+    n->net->use_graph = enabled != 0;
+    return 0;
+}
+
+int nbl_net_graph_active(nbl_net *n) { return n ? (n->net->graph_active() ? 1 : 0) : -1; }
 
 void *nbl_net_ctx(nbl_net *n) { return n ? (void*)n->net->ctx : NULL; }
 

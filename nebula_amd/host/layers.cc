@@ -394,9 +394,11 @@ void softmax_layer_t::init(section_config_t) {
 void softmax_layer_t::_forward_() {
     nbl_check(network->ctx, nbl_softmax_fwd(network->ctx, input_dev(), output_data_dev, network->batch_size, input_size),
               "nbl_softmax_fwd");
-    if(copy_to_host)
-        nbl_check(network->ctx, nbl_d2h(network->ctx, output_data, output_data_dev,
-                                        sizeof(float) * (size_t)output_size * network->batch_size), "nbl_d2h(softmax)");
+    if(copy_to_host) {
+        const size_t bytes = sizeof(float) * (size_t)output_size * network->batch_size;
+        if(network->defer_host_copy) nbl_check(network->ctx, nbl_d2h_async(network->ctx, output_data, output_data_dev, bytes), "nbl_d2h_async(softmax)");
+        else nbl_check(network->ctx, nbl_d2h(network->ctx, output_data, output_data_dev, bytes), "nbl_d2h(softmax)");
+    }
 }
 
 // ---- dropout / cost --------------------------------------------------------------------------------

@@ -24,7 +24,7 @@ network_t::network_t() :
     run_type(UNDEFINED_RUN), num_threads(1),
     learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
     input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
-    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1), defer_host_copy(false),
     input_layer(NULL), output_layer(NULL), num_layers(0) {}
 
 network_t::~network_t() {}
@@ -66,9 +66,10 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), last_step_only(false), fuse_shortcut(false),
+    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), last_step_only(false), fuse_shortcut(false), use_graph(false),
     first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false), image_staging_dev(NULL),
-    tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL), image_staging_bytes(0) {
+    tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL), image_staging_bytes(0),
+    graph_exec(NULL), graph_key(0), warm_key(0), graph_epoch(1), graph_unusable(false) {
     run_type = TEST_RUN;
     if(device < 0) return;            // dry run: shapes, cfg and .wgh handling only; no device, no forward
     int rc = nbl_ctx_create(device, &ctx);
@@ -80,6 +81,7 @@ inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
 }
 
 inference_net_t::~inference_net_t() {
+    if(graph_exec) { if(ctx) nbl_sync(ctx); (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec); }
     for(size_t i = layers.size(); i > 0; i--) delete layers[i - 1];
     for(size_t i = 0; i < events.size(); i++) (void)hipEventDestroy((hipEvent_t)events[i]);
     if(input_data_dev && ctx) nbl_free(ctx, input_data_dev);
@@ -123,6 +125,7 @@ void inference_net_t::build(config_t &config) {
             sc.get_setting("channels", &input_channel);
             sc.get_setting("batch", &batch_size);
             sc.get_setting("fuse_shortcut", &fuse_shortcut);
+            sc.get_setting("hip_graph", &use_graph);
             if(sc.exists("conv_split")) { unsigned v = 0; sc.get_setting("conv_split", &v); conv_split = v ? 1 : 0; }
             if(batch_override) batch_size = batch_override;
             input_size = input_height * input_width * input_channel;
@@ -271,9 +274,75 @@ void inference_net_t::run_layer(unsigned i) {
     if(producer) producer->output_data_dev = saved;
 }
 
-void inference_net_t::forward() {
+void inference_net_t::forward_eager() {
     if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     for(unsigned i = 0; i < num_layers; i++) run_layer(i);
+}
+
+void inference_net_t::invalidate_graph() {
+    ++graph_epoch;
+    if(graph_exec) {
+        if(ctx) nbl_sync(ctx);
+        (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+        graph_exec = NULL;
+    }
+}
+
+// What a pass launches depends on: the rows per pass, dense or token input, last_step_only, which softmax layers
+// copy to the host, and everything invalidate_graph() stands for (weights, plans).  Never 0.
+unsigned long long inference_net_t::pass_key() const {
+    unsigned long long k = 1469598103934665603ull;
+    const unsigned long long parts[] = { batch_size, time_step, (unsigned long long)last_step_only, graph_epoch,
+                                         (unsigned long long)(size_t)input_tokens_dev, (unsigned long long)(size_t)input_data_dev };
+    for(size_t i = 0; i < sizeof(parts) / sizeof(parts[0]); i++) k = (k ^ parts[i]) * 1099511628211ull;
+    for(unsigned i = 0; i < num_layers; i++)
+        if(layers[i]->layer_type == SOFTMAX_LAYER)
+            k = (k ^ (static_cast<const softmax_layer_t*>(layers[i])->copy_to_host ? 2u : 1u)) * 1099511628211ull;
+    return k ? k : 1;
+}
+
+void inference_net_t::forward() {
+    if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
+    if(!use_graph || graph_unusable) { forward_eager(); return; }
+    hipStream_t stream = (hipStream_t)nbl_ctx_stream(ctx);
+    const unsigned long long key = pass_key();
+    if(graph_exec && key != graph_key) invalidate_graph();      // (bumps the epoch: the key is taken again below)
+    const unsigned long long now = pass_key();
+    if(!graph_exec) {
+        if(warm_key != now) {          // first pass of this configuration: tile search, workspaces, lazily built tables
+            forward_eager();
+            warm_key = now;
+            return;
+        }
+        // second pass: record.  Nothing below may wait for the stream or allocate; a layer that does makes the
+        // recording fail, and the network stays on eager passes.
+        hipGraph_t graph = NULL;
+        if(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+            (void)hipGetLastError(); graph_unusable = true; forward_eager(); return;
+        }
+        defer_host_copy = true;
+        bool recorded = true;
+        try { for(unsigned i = 0; i < num_layers; i++) run_layer(i); }
+        catch(...) { recorded = false; }
+        defer_host_copy = false;
+        if(hipStreamEndCapture(stream, &graph) != hipSuccess || !graph) recorded = false;
+        hipGraphExec_t exec = NULL;
+        if(recorded && hipGraphInstantiate(&exec, graph, NULL, NULL, 0) != hipSuccess) recorded = false;
+        if(graph) (void)hipGraphDestroy(graph);
+        if(!recorded) {
+            (void)hipGetLastError();
+            graph_unusable = true;
+            forward_eager();
+            return;
+        }
+        graph_exec = (void*)exec;
+        graph_key = now;
+    }
+    if(hipGraphLaunch((hipGraphExec_t)graph_exec, stream) != hipSuccess)
+        throw std::runtime_error("Error: hipGraphLaunch failed");
+    // the recorded pass queues its host copies instead of waiting for each: wait once, as an eager pass ending in
+    // a softmax layer does
+    nbl_check(ctx, nbl_sync(ctx), "nbl_sync");
 }
 
 void inference_net_t::forward_timed(std::vector<float> &ms) {

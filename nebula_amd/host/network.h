@@ -54,6 +54,9 @@ public:
     // the patch rows between blocks, 1 = wherever the cost model says so; absent = measured per layer on
     // first use.  With 0 a convolution's result does not depend on the tile shape the search picks.
     int conv_split;
+    // Set while inference_net_t::forward() records or replays a HIP graph: a layer that copies to the host queues
+    // the copy on the stream instead of waiting for it, and forward() waits once at its end.
+    bool defer_host_copy;
 
     // Opens the headerless fp32 .wgh stream and lets every layer read its fields in cfg order
     // (models/networks/network.cc:99-122).
@@ -110,6 +113,16 @@ public:
     // [shortcut] computes the residual add and the shortcut's activation in its own epilogue.  Same float
     // operations in the same order; the convolution's pre-shortcut output is then never materialised.
     bool fuse_shortcut;
+    // [net] key `hip_graph=1` (a key the reference ignores): forward() records the launches of one pass into a
+    // HIP graph and replays it from then on, so a pass costs one launch on the host instead of one per kernel
+    // (recurrent nets launch a kernel per layer and time step).  The first pass of a configuration runs
+    // eagerly (tile search, workspaces grow), the second is recorded, later ones replay.  Anything that changes
+    // what a pass launches (weights, token vs. dense input, last_step_only, the softmax copy) makes the next
+    // pass start over; call invalidate_graph() after changing a layer behind the network's back.
+    bool use_graph;
+    void invalidate_graph();
+    bool graph_active() const { return graph_exec != NULL; }   // true once a recorded pass is being replayed
+    void forward_eager();
 
 protected:
     void init_network(const std::string m_network_config);
@@ -127,6 +140,11 @@ private:
     unsigned *tokens_dev, *labels_dev; float *cost_dev;   // token input, label tokens and the device-side sum
     size_t image_staging_bytes;
     std::vector<void*> events;
+    void *graph_exec;                   // hipGraphExec_t of the recorded pass, NULL if none
+    unsigned long long graph_key, warm_key;   // configuration the graph was recorded for / the last eager pass ran with
+    unsigned graph_epoch;               // bumped by invalidate_graph()
+    bool graph_unusable;                // recording failed once: stay eager
+    unsigned long long pass_key() const;
 };
 
 // Throws std::runtime_error(nbl_last_error) when an ABI call fails.

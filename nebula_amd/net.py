@@ -36,6 +36,8 @@ SIGNATURES = {
     "nbl_net_layer_output": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
     "nbl_net_pool_index": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
     "nbl_net_softmax_copy": (C.c_int, [_vp, C.c_int]),
+    "nbl_net_set_graph": (C.c_int, [_vp, C.c_int]),
+    "nbl_net_graph_active": (C.c_int, [_vp]),
     "nbl_net_ctx": (_vp, [_vp]),
 }
 
@@ -179,6 +181,14 @@ class Network:
 
     def softmax_copy(self, enabled):
         lib().nbl_net_softmax_copy(self.h, 1 if enabled else 0)
+
+    def set_graph(self, enabled):
+        """Record one forward pass into a HIP graph and replay it from then on (first pass eager, second recorded)."""
+        lib().nbl_net_set_graph(self.h, 1 if enabled else 0)
+
+    @property
+    def graph_active(self):
+        return lib().nbl_net_graph_active(self.h) == 1
 
     @property
     def ctx(self):
