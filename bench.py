@@ -183,16 +183,24 @@ def image_input(args):
 
 def recurrent_driver(args):
     """The recurrent driver's test step (models/networks/recurrent.cc): one-hot words of a 10000-word vocabulary,
-    T = 64 steps x `batch` sequences, 2 x LSTM 1024, projection + softmax on every row, perplexity update.
-    Timed twice: one-hot rows as token indices (gather), and as the dense [T*B x 10000] matrix the reference builds."""
+    T = 64 steps x `batch` sequences, 2 x LSTM 1024, projection + softmax on every row, perplexity update
+    (--recurrent-net rnn: rnn_large's shape instead, 5 normalised RNN layers of 1024, T = 40, 8713 words, batch 32).
+    Timed twice: one-hot rows as token indices (gather), and as the dense [T*B x V] matrix the reference builds."""
     from nebula_amd import zoo
     from nebula_amd.net import Network
-    B = args.batch or 64
-    T, V, H = 64, 10000, 1024
     rng = np.random.default_rng(5)
-    cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=2, classes=V)
-    net = Network(cfg)
-    net.load_weight_blob(make_weights(net.weight_layout(), rng, "lstm"))
+    if args.recurrent_net == "rnn":
+        B = args.batch or 32
+        T, V, H = 40, 8713, 1024
+        cfg = zoo.rnn_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=5)
+        net = Network(cfg)
+        net.load_weight_blob(make_weights(net.weight_layout(), rng, "he"))
+    else:
+        B = args.batch or 64
+        T, V, H = 64, 10000, 1024
+        cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=2, classes=V)
+        net = Network(cfg)
+        net.load_weight_blob(make_weights(net.weight_layout(), rng, "lstm"))
     net.softmax_copy(False)              # the probabilities stay on the device; the perplexity sum is computed there
     tokens = rng.integers(0, V, (T, B)).astype(np.uint32)
     labels = np.roll(tokens.ravel(), -1).reshape(T, B)
@@ -219,7 +227,8 @@ def recurrent_driver(args):
                      "layer_ms": [round(float(v), 3) for v in layer_ms], "perplexity_figure": round(float(ppl), 2)}
         log(mode, out[mode])
     net.close()
-    print(json.dumps({"metric": "recurrent driver step (PTB shape) sequences/s", "value": out["tokens"]["sequences_per_s"],
+    print(json.dumps({"metric": "recurrent driver step (%s) sequences/s" % ("rnn_large shape" if args.recurrent_net == "rnn" else "PTB shape"),
+                      "value": out["tokens"]["sequences_per_s"],
                       "unit": "sequences/s", "batch": B, "time_steps": T, "vocabulary": V, "steps": args.steps,
                       "tokens": out["tokens"], "dense_one_hot": out["dense one-hot"]}), flush=True)
 
@@ -239,6 +248,7 @@ def main():
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--recurrent-net", default="lstm", choices=["lstm", "rnn"], help="network of --workload ptb")
     ap.add_argument("--graph", type=int, default=0, help="1: forward passes are replays of a recorded HIP graph, 0 (default): eager "
                     "launches (the passes are GPU-bound on this machine: both take the same time)")
     args = ap.parse_args()

@@ -192,6 +192,11 @@ int nbl_rnn_pack(nbl_ctx *ctx, const float *const *weight_host, const float *con
                  const float *const *scale_host, const float *const *mean_host, const float *const *var_host,
                  unsigned I, unsigned O, int act, nbl_rnn_plan **out);
 int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *plan, const float *x_dev, float *y_dev, unsigned T, unsigned B);
+/* The same layer fed by the recurrent driver's one-hot rows (models/networks/recurrent.cc:179-204) given as the
+ * position of their 1.0, tokens_dev[T*B] time-major, as nbl_lstm_fwd_tokens: the input gate's product becomes a
+ * gather of rows of the transposed weights (built on first use), with the gate's own scale, bias and activation.
+ * Same values as nbl_rnn_fwd on the one-hot matrix; a token >= I stands for an all-zero row. */
+int nbl_rnn_fwd_tokens(nbl_ctx *ctx, nbl_rnn_plan *plan, const unsigned *tokens_dev, float *y_dev, unsigned T, unsigned B);
 int nbl_rnn_plan_destroy(nbl_ctx *ctx, nbl_rnn_plan *plan);
 
 /* count_dev[0] = number of rows whose label is among the k largest entries of probs[row][0..n): the

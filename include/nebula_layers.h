@@ -53,8 +53,8 @@ int nbl_net_set_input(nbl_net *net, const float *host, size_t count);
  * INTER_LINEAR), scaled by 1/255 and stored as planes with planes 0 and 2 swapped. */
 int nbl_net_set_input_images(nbl_net *net, const unsigned char *host, unsigned images, unsigned height, unsigned width);
 /* recurrent_t::load_data() (models/networks/recurrent.cc:179-204) without the one-hot matrix: tokens[T*B]
- * (time-major; = batch_size entries) name the position of the 1.0 in each input row.  Needs an [lstm] as the
- * first layer, which then gathers weight columns instead of multiplying.  nbl_net_set_input switches back. */
+ * (time-major; = batch_size entries) name the position of the 1.0 in each input row.  Needs an [lstm] or an
+ * [rnn] as the first layer, which then gathers weight columns instead of multiplying.  nbl_net_set_input switches back. */
 int nbl_net_set_input_tokens(nbl_net *net, const unsigned *host, size_t count);
 /* recurrent_t::print_results(), test branch (recurrent.cc:239-247): after a forward, adds the output layer's
  * probabilities of the label tokens (one per output row) to the running sum and returns the driver's figure

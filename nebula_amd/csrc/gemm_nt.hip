@@ -697,19 +697,32 @@ __global__ void transpose_kernel(const float *__restrict__ src, float *__restric
 // token[row] of its transpose, so the [T*B x V].[V x 4H] product becomes a gather of T*B rows:
 //   gx[row][n] = sub_act(UcatT[token[row]][n] + bu[n])
 // (the same single float add the GEMM epilogue performs on a sum whose other terms are zero).
-__global__ void lstm_token_gather_kernel(const float *__restrict__ ucat_t, const unsigned *__restrict__ tokens,
-                                         const float *__restrict__ bu, float *__restrict__ gx,
-                                         unsigned Np, unsigned vocab, int sub_act) {
+__global__ void token_gather_kernel(const float *__restrict__ w_t, const unsigned *__restrict__ tokens,
+                                    const float *__restrict__ scale, const float *__restrict__ bias,
+                                    float *__restrict__ out_rows, unsigned Np, unsigned vocab, int act) {
+    // scale: per-column factor of a sub-layer with folded batch normalisation (the epilogue form of the products:
+    // v * g + b), or NULL (v + b)
     const unsigned row = blockIdx.x, tok = tokens[row];
-    const float4 *__restrict__ src = reinterpret_cast<const float4*>(ucat_t + (size_t)tok * Np);
-    const float4 *__restrict__ b4 = reinterpret_cast<const float4*>(bu);
-    float4 *__restrict__ out = reinterpret_cast<float4*>(gx + (size_t)row * Np);
-    for(unsigned i = threadIdx.x; i < Np / 4; i += blockDim.x) {
-        float4 v = tok < vocab ? src[i] : make_float4(0.f, 0.f, 0.f, 0.f);     // a token outside the vocabulary is an all-zero row
-        const float4 b = b4[i];
-        v.x = nbl_act_apply(sub_act, v.x + b.x); v.y = nbl_act_apply(sub_act, v.y + b.y);
-        v.z = nbl_act_apply(sub_act, v.z + b.z); v.w = nbl_act_apply(sub_act, v.w + b.w);
-        out[i] = v;
+    const float *__restrict__ src = w_t + (size_t)tok * Np;
+    float *__restrict__ out = out_rows + (size_t)row * Np;
+    if((Np & 3u) == 0) {
+        for(unsigned i = threadIdx.x; i < Np / 4; i += blockDim.x) {
+            // a token outside the vocabulary is an all-zero row
+            const float4 q = tok < vocab ? reinterpret_cast<const float4*>(src)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 b = reinterpret_cast<const float4*>(bias)[i];
+            float v[4] = { q.x, q.y, q.z, q.w };
+            const float bb[4] = { b.x, b.y, b.z, b.w };
+            float gg[4] = { 1.f, 1.f, 1.f, 1.f };
+            if(scale) { const float4 g = reinterpret_cast<const float4*>(scale)[i]; gg[0] = g.x; gg[1] = g.y; gg[2] = g.z; gg[3] = g.w; }
+            #pragma unroll
+            for(int c = 0; c < 4; c++) v[c] = nbl_act_apply(act, scale ? v[c] * gg[c] + bb[c] : v[c] + bb[c]);
+            reinterpret_cast<float4*>(out)[i] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    } else {
+        for(unsigned i = threadIdx.x; i < Np; i += blockDim.x) {
+            const float v = tok < vocab ? src[i] : 0.0f;
+            out[i] = nbl_act_apply(act, scale ? v * scale[i] + bias[i] : v + bias[i]);
+        }
     }
 }
 
@@ -745,6 +758,7 @@ struct nbl_rnn_plan {
     float *in_all, *states, *hid0, *tmp;     // [T*B][O], [T*B][O], [B][O], [B][O]
     float *wh_op;                            // hidden gate's weights in operand-major layout (O % 128 == 0)
     float *sop[2]; size_t sop_bytes;         // state of the previous / this step in operand-major layout
+    float *wi_t;                             // input gate's weights transposed to [I][O], built on the first token-fed pass
     size_t rows_alloc, seqs_alloc;
 };
 
@@ -1034,9 +1048,9 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
                                p->ucat_dev, p->ucat_t_dev, Np, p->I);
             NBL_LAUNCH_CHECK(ctx, "transpose_kernel");
         }
-        hipLaunchKernelGGL(lstm_token_gather_kernel, dim3(T * B), dim3(256), 0, ctx->stream,
-                           p->ucat_t_dev, tokens_dev, p->bu_dev, p->gx_dev, Np, p->I, p->sub_act);
-        NBL_LAUNCH_CHECK(ctx, "lstm_token_gather_kernel");
+        hipLaunchKernelGGL(token_gather_kernel, dim3(T * B), dim3(256), 0, ctx->stream,
+                           p->ucat_t_dev, tokens_dev, (const float*)NULL, p->bu_dev, p->gx_dev, Np, p->I, p->sub_act);
+        NBL_LAUNCH_CHECK(ctx, "token_gather_kernel");
     } else if((rc = launch_fc(ctx, x_dev, p->ucat_dev, p->gx_dev, (int)(T * B), (int)Np, (int)p->I, NULL, p->bu_dev,
                               p->sub_act, 0, NULL, NULL)) != NBL_OK) return rc;
     const size_t step = (size_t)B * p->H;
@@ -1155,17 +1169,17 @@ int nbl_rnn_plan_destroy(nbl_ctx *ctx, nbl_rnn_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     for(int s = 0; s < 3; s++) if(p->gate[s]) nbl_fc_plan_destroy(ctx, p->gate[s]);
     nbl_free(ctx, p->in_all); nbl_free(ctx, p->states); nbl_free(ctx, p->hid0); nbl_free(ctx, p->tmp);
-    nbl_free(ctx, p->wh_op); nbl_free(ctx, p->sop[0]); nbl_free(ctx, p->sop[1]);
+    nbl_free(ctx, p->wh_op); nbl_free(ctx, p->sop[0]); nbl_free(ctx, p->sop[1]); nbl_free(ctx, p->wi_t);
     delete p;
     return NBL_OK;
 }
 
-int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev, unsigned T, unsigned B) {
-    if(!ctx) return NBL_EINVAL;
-    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_rnn_fwd: NULL argument");
+// x_dev: dense input rows, or NULL with tokens_dev: the position of the single 1.0 of each one-hot row
+static int rnn_forward(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, const unsigned *tokens_dev, float *y_dev,
+                       unsigned T, unsigned B) {
     if(T == 0 || B == 0) return NBL_OK;
     const size_t rows = (size_t)T * B;
-    if(rows * p->O >= (1ull << 31) || rows * p->I >= (1ull << 31))
+    if(rows * p->O >= (1ull << 31) || (x_dev && rows * p->I >= (1ull << 31)))
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_rnn_fwd: tensors of 2^31 elements or more are not supported");
     int rc;
     if(p->rows_alloc < rows || p->seqs_alloc < B) {
@@ -1180,8 +1194,20 @@ int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev,
     }
     nbl_fc_plan *gi = p->gate[0], *gh = p->gate[1], *go = p->gate[2];
     // input gate for every step at once: it does not depend on the recurrence
-    if((rc = launch_fc(ctx, x_dev, gi->w_dev, p->in_all, (int)rows, (int)p->O, (int)p->I, gi->g_dev, gi->b_dev,
-                       gi->act, gi->has_scale, &gi->ws_dev, &gi->ws_bytes, gi->w_tiled_dev)) != NBL_OK) return rc;
+    if(tokens_dev) {
+        // one-hot rows: the product is column token[row] of the weights, i.e. a row of their transpose
+        if(!p->wi_t) {
+            if((rc = nbl_malloc(ctx, (void**)&p->wi_t, (size_t)p->O * p->I * sizeof(float))) != NBL_OK) return rc;
+            hipLaunchKernelGGL(transpose_kernel, dim3(nbl_div_up(p->I, 32), nbl_div_up(p->O, 32)), dim3(256), 0, ctx->stream,
+                               gi->w_dev, p->wi_t, p->O, p->I);
+            NBL_LAUNCH_CHECK(ctx, "transpose_kernel");
+        }
+        hipLaunchKernelGGL(token_gather_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream,
+                           p->wi_t, tokens_dev, gi->has_scale ? gi->g_dev : (const float*)NULL, gi->b_dev, p->in_all,
+                           p->O, p->I, gi->act);
+        NBL_LAUNCH_CHECK(ctx, "token_gather_kernel");
+    } else if((rc = launch_fc(ctx, x_dev, gi->w_dev, p->in_all, (int)rows, (int)p->O, (int)p->I, gi->g_dev, gi->b_dev,
+                              gi->act, gi->has_scale, &gi->ws_dev, &gi->ws_bytes, gi->w_tiled_dev)) != NBL_OK) return rc;
     const size_t step = (size_t)B * p->O;
     const bool one_launch = p->wh_op != NULL && aligned16(p->in_all) && aligned16(p->states) && aligned16(p->hid0);
     if(one_launch) {
@@ -1227,6 +1253,18 @@ int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev,
     if(T > 1 && (rc = launch_fc(ctx, p->states + step, go->w_dev, y_dev + step, (int)(rows - B), (int)p->O, (int)p->O,
                                 go->g_dev, go->b_dev, go->act, go->has_scale, &go->ws_dev, &go->ws_bytes, go->w_tiled_dev)) != NBL_OK) return rc;
     return NBL_OK;
+}
+
+int nbl_rnn_fwd(nbl_ctx *ctx, nbl_rnn_plan *p, const float *x_dev, float *y_dev, unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && x_dev && y_dev, "nbl_rnn_fwd: NULL argument");
+    return rnn_forward(ctx, p, x_dev, NULL, y_dev, T, B);
+}
+
+int nbl_rnn_fwd_tokens(nbl_ctx *ctx, nbl_rnn_plan *p, const unsigned *tokens_dev, float *y_dev, unsigned T, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && tokens_dev && y_dev, "nbl_rnn_fwd_tokens: NULL argument");
+    return rnn_forward(ctx, p, NULL, tokens_dev, y_dev, T, B);
 }
 
 }  // extern "C"

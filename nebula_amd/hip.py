@@ -41,6 +41,7 @@ SIGNATURES = {
     "nbl_lstm_fwd_tokens": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
     "nbl_rnn_pack": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_rnn_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u]),
+    "nbl_rnn_fwd_tokens": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u]),
     "nbl_rnn_plan_destroy": (C.c_int, [_vp, _vp]),
     "nbl_topk_matches": (C.c_int, [_vp, _vp, _vp, _u, _u, _u, _vp]),
     "nbl_target_prob_sum": (C.c_int, [_vp, _vp, _vp, _u, _u, _vp]),

@@ -600,6 +600,13 @@ void rnn_layer_t::pack() {
 
 void rnn_layer_t::_forward_() {
     if(!plan) throw std::runtime_error("Error: rnn layer has no weights (init_weight not called)");
+    if(!prev_layer && network->input_tokens_dev) {      // one-hot input rows given as token indices
+        nbl_check(network->ctx,
+                  nbl_rnn_fwd_tokens(network->ctx, plan, network->input_tokens_dev, output_data_dev, network->time_step,
+                                     network->batch_size / network->time_step),
+                  "nbl_rnn_fwd_tokens");
+        return;
+    }
     nbl_check(network->ctx,
               nbl_rnn_fwd(network->ctx, plan, input_dev(), output_data_dev, network->time_step,
                           network->batch_size / network->time_step),

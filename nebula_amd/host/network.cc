@@ -188,8 +188,8 @@ void inference_net_t::set_input_tokens(const unsigned *host, size_t count) {
     if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
     if(!is_recurrent) throw std::runtime_error("Error: token input on a network without time_steps");
     if(count != (size_t)batch_size) throw std::runtime_error("Error: token input has the wrong size");
-    if(layers.empty() || layers[0]->layer_type != LSTM_LAYER)
-        throw std::runtime_error("Error: token input needs an lstm layer first");
+    if(layers.empty() || (layers[0]->layer_type != LSTM_LAYER && layers[0]->layer_type != RNN_LAYER))
+        throw std::runtime_error("Error: token input needs an lstm or rnn layer first");
     if(!tokens_dev) nbl_check(ctx, nbl_malloc(ctx, (void**)&tokens_dev, (size_t)batch_size * sizeof(unsigned)), "nbl_malloc(tokens)");
     nbl_check(ctx, nbl_h2d(ctx, tokens_dev, host, count * sizeof(unsigned)), "nbl_h2d(tokens)");
     input_tokens_dev = tokens_dev;

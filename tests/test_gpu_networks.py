@@ -313,6 +313,47 @@ def test_recurrent_driver_contract_tokens_and_perplexity():
         np.testing.assert_array_equal(net.output(0).view(np.uint32), dense[0].view(np.uint32))
 
 
+@pytest.mark.parametrize("H,V", [(128, 40), (96, 37)])
+def test_rnn_token_input_equals_one_hot_input(H, V):
+    """rnn_large's shape in small: normalised [rnn] layers fed by the recurrent driver's one-hot rows.  Token input
+    (a gather of input-gate weight columns) must equal the dense one-hot product bit for bit, for the one-launch
+    step kernel (width 128) and the general path (width 96, odd vocabulary), and match the oracle."""
+    from nebula_amd import zoo
+    from nebula_amd.net import Network
+    print("CASE rnn tokens", H, V, flush=True)
+    T, B = 5, 6
+    rng = np.random.default_rng(H + V)
+    cfg = zoo.rnn_cfg(batch=B, time_steps=T, input_size=V, hidden=H, layers=2)
+    onet = ob.OracleNet(cfg)
+    blob = _random_weights(onet.specs, rng)
+    onet.load_weights(blob)
+    tokens = rng.integers(0, V, (T, B)).astype(np.uint32)
+    x = np.zeros((T, B, V), np.float32)
+    x[np.arange(T)[:, None], np.arange(B)[None, :], tokens] = 1.0
+    ob.use_custom_gemm()
+    want = onet.forward(x)
+    with Network(cfg) as net:
+        net.load_weight_blob(blob)
+        net.set_input(x)
+        net.forward()
+        dense = [net.output(i) for i in range(net.num_layers)]
+        net.set_input_tokens(tokens)
+        net.forward()
+        tok = [net.output(i) for i in range(net.num_layers)]
+        for i, (u, v) in enumerate(zip(dense, tok)):
+            np.testing.assert_array_equal(u.view(np.uint32), v.view(np.uint32), err_msg="layer %d" % i)
+            assert rel(v, want[i].ravel()) <= TOL, (i, rel(v, want[i].ravel()))
+        # a token outside the vocabulary is an all-zero input row
+        tokens2 = tokens.copy(); tokens2[1, 2] = V + 3
+        x2 = x.copy(); x2[1, 2, :] = 0.0
+        net.set_input(x2)
+        net.forward()
+        d2 = net.output(0)
+        net.set_input_tokens(tokens2)
+        net.forward()
+        np.testing.assert_array_equal(net.output(0).view(np.uint32), d2.view(np.uint32))
+
+
 def test_image_driver_topk_count(golden_dir):
     """Running top-k match count of the image driver on the DBN fixture's probabilities."""
     from nebula_amd.net import Network
