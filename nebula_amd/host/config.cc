@@ -36,7 +36,12 @@ void section_config_t::add_setting(std::string m_key, std::string m_value) {
     settings.insert(std::make_pair(lowercase(m_key), lowercase(m_value)));   // insert: first one wins
 }
 
-bool section_config_t::exists(std::string m_key) { return settings.count(lowercase(m_key)) != 0; }
+const std::string *section_config_t::find(std::string &m_key) const {
+    const std::map<std::string, std::string>::const_iterator at = settings.find(lowercase(m_key));
+    return at == settings.end() ? NULL : &at->second;
+}
+
+bool section_config_t::exists(std::string m_key) { return find(m_key) != NULL; }
 
 void config_t::parse(std::string m_config_name) {
     std::ifstream in(m_config_name.c_str());

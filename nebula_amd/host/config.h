@@ -15,22 +15,26 @@ namespace nebula {
 
 std::string &lowercase(std::string &s);
 
+// One "[name]" block of a cfg file: its key=value lines.
 class section_config_t {
 public:
+    std::string name;
+
     explicit section_config_t(std::string m_name);
     void add_setting(std::string m_key, std::string m_value);
     bool exists(std::string m_key);
+    // *m_var = the value of m_key read with operator>>; false (and *m_var untouched) when the key is absent
     template <typename T>
     bool get_setting(std::string m_key, T *m_var) {
-        std::map<std::string, std::string>::iterator it = settings.find(lowercase(m_key));
-        if(it == settings.end()) return false;
-        std::stringstream ss(it->second);
-        ss >> *m_var;
+        const std::string *text = find(m_key);
+        if(!text) return false;
+        std::istringstream in(*text);
+        in >> *m_var;
         return true;
     }
-    std::string name;
 
 private:
+    const std::string *find(std::string &m_key) const;     // lower-cases m_key first, as every access does
     std::map<std::string, std::string> settings;
 };
 
