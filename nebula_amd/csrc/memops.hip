@@ -248,8 +248,60 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// One block of THREADS threads per row (long rows take 1024 threads: the exp is double precision and
-// there are only as many blocks as rows).
+// Rows of up to THREADS * PER entries: a thread keeps its PER entries (columns tid, tid + THREADS, ...) in
+// registers, so the row is read once and written once; maximum, partial sums and their trees are those of the
+// general kernel below, and so is every result bit.
+template<int THREADS, int PER>
+__global__ __launch_bounds__(THREADS) void softmax_row_in_registers_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
+    constexpr int WAVES = THREADS / 64;
+    __shared__ float red[WAVES];
+    const float *in = x + (size_t)blockIdx.x * n;
+    float *out = y + (size_t)blockIdx.x * n;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    float v[PER];
+    float m = -FLT_MAX;
+    #pragma unroll
+    for(int i = 0; i < PER; i++) {
+        const unsigned j = tid + i * THREADS;
+        v[i] = j < n ? in[j] : -FLT_MAX;
+        m = fmaxf(m, v[i]);
+    }
+    m = wave_max(m);
+    if(lane == 0) red[wave] = m;
+    __syncthreads();
+    m = red[0];
+    #pragma unroll
+    for(int w = 1; w < WAVES; w++) m = fmaxf(m, red[w]);
+    __syncthreads();
+    float s = 0.0f;
+    #pragma unroll
+    for(int i = 0; i < PER; i++) {
+        const unsigned j = tid + i * THREADS;
+        if(j < n) {
+            v[i] = (float)exp((double)(v[i] - m));
+            s += v[i];
+        }
+    }
+    s = wave_sum(s);
+    if(lane == 0) red[wave] = s;
+    __syncthreads();
+    float part[WAVES];
+    #pragma unroll
+    for(int w = 0; w < WAVES; w++) part[w] = red[w];
+    #pragma unroll
+    for(int width = WAVES / 2; width >= 1; width /= 2)
+        #pragma unroll
+        for(int w = 0; w < width; w++) part[w] = part[2 * w] + part[2 * w + 1];
+    s = part[0];
+    #pragma unroll
+    for(int i = 0; i < PER; i++) {
+        const unsigned j = tid + i * THREADS;
+        if(j < n) out[j] = v[i] / s;
+    }
+}
+
+// One block of THREADS threads per row of any length (long rows take 1024 threads: the exp is double precision and
+// there are only as many blocks as rows); the row is read three times and written twice.
 template<int THREADS>
 __global__ __launch_bounds__(THREADS) void softmax_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
     constexpr int WAVES = THREADS / 64;
@@ -541,8 +593,10 @@ int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned row
     if(!ctx) return NBL_EINVAL;
     NBL_REQUIRE(ctx, x_dev && y_dev, "nbl_softmax_fwd: NULL pointer");
     if(rows == 0 || n == 0) return NBL_OK;
-    if(n > 2048) hipLaunchKernelGGL(softmax_kernel<1024>, dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
-    else         hipLaunchKernelGGL(softmax_kernel<256>, dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    if(n <= 1024)       hipLaunchKernelGGL((softmax_row_in_registers_kernel<256, 4>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    else if(n <= 2048)  hipLaunchKernelGGL((softmax_row_in_registers_kernel<256, 8>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    else if(n <= 16384) hipLaunchKernelGGL((softmax_row_in_registers_kernel<1024, 16>), dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
+    else                hipLaunchKernelGGL(softmax_kernel<1024>, dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
     NBL_LAUNCH_CHECK(ctx, "softmax_kernel");
     return NBL_OK;
 }

@@ -359,7 +359,9 @@ def test_bias_and_batchnorm_primitives(ctx):
     assert rel(got, a) <= 1e-6
 
 
-@pytest.mark.parametrize("shape", [(6, 333), (64, 1000), (3, 10000), (1, 5), (128, 1000)])
+# row lengths either side of every kernel choice (4, 8 or 16 entries per thread in registers, then the general kernel)
+@pytest.mark.parametrize("shape", [(6, 333), (64, 1000), (3, 10000), (1, 5), (128, 1000), (2, 1024), (2, 1025), (3, 2048),
+                                   (2, 2049), (2, 8713), (2, 16384), (2, 16385), (3, 20000), (5, 1)])
 def test_softmax(ctx, shape):
     announce("softmax", shape)
     rng = np.random.default_rng(shape[1])
@@ -369,6 +371,11 @@ def test_softmax(ctx, shape):
     assert rel(got, want) <= TOL
     np.testing.assert_array_equal(got.argmax(1), want.argmax(1))
     assert np.abs(got.sum(1) - 1).max() < 1e-5
+    # closed form in double, and shift invariance (the row maximum is subtracted first)
+    e = np.exp(x.astype(np.float64) - x.astype(np.float64).max(1, keepdims=True))
+    assert np.abs(got - e / e.sum(1, keepdims=True)).max() <= 2e-6
+    shifted = ctx.softmax(ctx.array(x + np.float32(8.0))).numpy()
+    assert np.abs(shifted - got).max() <= 2e-6
 
 
 LSTM = [(3, 2, 5, 4, False, "linear"), (4, 3, 6, 5, True, "tanh"), (6, 8, 64, 96, False, "linear"),
