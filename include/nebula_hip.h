@@ -147,6 +147,15 @@ int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
                 unsigned I, unsigned O, int act, nbl_fc_plan **out);
 int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B);
 int nbl_fc_plan_destroy(nbl_ctx *ctx, nbl_fc_plan *plan);
+/* nbl_fc_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels, same split of the
+ * fan-in and therefore the same bits as nbl_fc_fwd, but the split-K partial sums go to a static device array of
+ * NBL_FC_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends, and the call
+ * never allocates or frees.  A product whose partial sums (splits x B x O floats; the split count is at most 64
+ * and falls as B x O grows) exceed the array is refused with NBL_EUNSUPPORTED.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race. */
+#define NBL_FC_NOALLOC_SCRATCH_BYTES (16u << 20)
+int nbl_fc_fwd_noalloc(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B);
 
 /* ---- LSTM --------------------------------------------------------------------------------------
  * nbl_lstm_pack: lstm_layer_t::init_weight() (models/layers/lstm_layer.cc:194-206).  The eight

@@ -19,6 +19,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -765,9 +766,12 @@ struct nbl_rnn_plan {
 namespace {
 
 // Bw_tiled: the same weights as 16 KB tiles (see GemmArgs::b_tiled), or NULL; used whenever the buffer-load kernel runs
+// ws / ws_bytes: the plan's split-K workspace, grown here on demand (NULL: never split).  With fixed_ws the partial
+// sums go to that buffer of fixed_cap bytes instead and nothing is allocated or freed: a product whose split
+// needs more than fixed_cap is refused.
 int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, int N, int K,
               const float *g, const float *b, int act, int has_scale, float **ws, size_t *ws_bytes,
-              const float *Bw_tiled = NULL) {
+              const float *Bw_tiled = NULL, float *fixed_ws = NULL, size_t fixed_cap = 0) {
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.A = A; a.Bw = Bw; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K; a.ldc = N;
@@ -784,7 +788,7 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     // 256 CUs (three on some, two on others) stream a 492 MB matrix 7 % slower than 500.
     int S = 1;
     const int ktiles = nbl_div_up(K, GEMM_BK);
-    if(ws) {
+    if(ws || fixed_ws) {
         double best = 0.0;
         for(int s = 1; s <= 64 && ktiles / s >= 2; s++) {
             const int chunk = nbl_div_up(ktiles, s), s_eff = nbl_div_up(ktiles, chunk);
@@ -804,14 +808,23 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     if(buf_ok && Bw_tiled) { a.Bw = Bw_tiled; a.b_tiled = 1; }
     if(S > 1) {
         const size_t need = (size_t)S * M * N * sizeof(float);
-        if(*ws_bytes < need) {
-            int rc = nbl_free(ctx, *ws);
-            *ws = NULL; *ws_bytes = 0;
-            if(rc != NBL_OK) return rc;
-            if((rc = nbl_malloc(ctx, (void**)ws, need)) != NBL_OK) return rc;
-            *ws_bytes = need;
+        float *part;
+        if(fixed_ws) {
+            if(need > fixed_cap)
+                return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: the %d partial sums of this %d x %d product need %zu bytes, "
+                                "the static scratch holds %zu", S, M, N, need, fixed_cap);
+            part = fixed_ws;
+        } else {
+            if(*ws_bytes < need) {
+                int rc = nbl_free(ctx, *ws);
+                *ws = NULL; *ws_bytes = 0;
+                if(rc != NBL_OK) return rc;
+                if((rc = nbl_malloc(ctx, (void**)ws, need)) != NBL_OK) return rc;
+                *ws_bytes = need;
+            }
+            part = *ws;
         }
-        a.C = *ws;
+        a.C = part;
         if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(buf_ok)                hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
@@ -823,12 +836,12 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(split-k)");
         const size_t total = (size_t)M * N;
-        if(N % 4 == 0 && aligned16(*ws) && aligned16(C))
+        if(N % 4 == 0 && aligned16(part) && aligned16(C))
             hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
-                               *ws, C, g, b, M, N, S, act, has_scale);
+                               (const float*)part, C, g, b, M, N, S, act, has_scale);
         else
             hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
-                               *ws, C, g, b, M, N, S, act, has_scale);
+                               (const float*)part, C, g, b, M, N, S, act, has_scale);
         NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
     } else {
         if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
@@ -916,6 +929,56 @@ int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float 
     nbl_fc_plan *p = const_cast<nbl_fc_plan*>(plan);   // the split-K workspace is a cache
     return launch_fc(ctx, x_dev, p->w_dev, y_dev, (int)B, (int)p->O, (int)p->I, p->g_dev, p->b_dev,
                      p->act, p->has_scale ? 1 : 0, &p->ws_dev, &p->ws_bytes, p->w_tiled_dev);
+}
+
+// ---- fully connected without allocation ----------------------------------------------------------
+// Split-K partial sums of nbl_fc_fwd_noalloc live in a file-scope device array, one copy per GPU for the life of
+// the process.  On the host the array's NAME is only a handle: the address kernels can use comes from
+// hipGetSymbolAddress, asked once per device with that device current, and is kept per device.
+}  // extern "C"
+
+namespace {
+
+constexpr size_t FC_SCRATCH_BYTES = (size_t)NBL_FC_NOALLOC_SCRATCH_BYTES;
+constexpr int FC_SCRATCH_MAX_DEVICES = 64;
+static __device__ __align__(256) float fc_noalloc_scratch[FC_SCRATCH_BYTES / sizeof(float)];
+float *g_fc_scratch_ptr[FC_SCRATCH_MAX_DEVICES];
+std::mutex g_fc_scratch_lock;
+
+// Device address of this GPU's copy of the scratch array (looked up on the first call for the device).
+int fc_scratch_address(nbl_ctx *ctx, float **out) {
+    if(ctx->device < 0 || ctx->device >= FC_SCRATCH_MAX_DEVICES)
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: device index %d beyond %d", ctx->device, FC_SCRATCH_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_fc_scratch_lock);
+    if(!g_fc_scratch_ptr[ctx->device]) {
+        NBL_HIP(ctx, hipSetDevice(ctx->device));
+        void *p = NULL;
+        NBL_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(fc_noalloc_scratch)));
+        if(!p || ((size_t)p & 255) != 0)
+            return nbl_fail(ctx, NBL_EHIP, "nbl_fc_fwd_noalloc: hipGetSymbolAddress returned an unusable address %p", p);
+        g_fc_scratch_ptr[ctx->device] = (float*)p;
+    }
+    *out = g_fc_scratch_ptr[ctx->device];
+    return NBL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nbl_fc_fwd_noalloc(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_fc_fwd_noalloc: NULL argument");
+    if(B == 0) return NBL_OK;
+    if((size_t)B * plan->I >= (1ull << 31) || (size_t)B * plan->O >= (1ull << 31))
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: tensors of 2^31 elements or more are not supported");
+    float *scratch = NULL;
+    const int rc = fc_scratch_address(ctx, &scratch);
+    if(rc != NBL_OK) return rc;
+    // every partial sum the reduction reads is written by this call's product kernel first, so the contents a
+    // previous call left behind never show
+    return launch_fc(ctx, x_dev, plan->w_dev, y_dev, (int)B, (int)plan->O, (int)plan->I, plan->g_dev, plan->b_dev,
+                     plan->act, plan->has_scale ? 1 : 0, NULL, NULL, plan->w_tiled_dev, scratch, FC_SCRATCH_BYTES);
 }
 
 // ---- LSTM ----------------------------------------------------------------------------------------
