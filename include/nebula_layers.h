@@ -69,9 +69,18 @@ int nbl_net_forward(nbl_net *net);
 int nbl_net_sync(nbl_net *net);
 /* forward with a HIP event between layers: ms[i] = duration of layer i (num_layers entries) */
 int nbl_net_forward_timed(nbl_net *net, float *ms);
-/* device -> host copy of layer's output ([batch_size][output_size]) or maxpool argmax table */
+/* device -> host copy of layer's output ([batch_size][output_size]).  A convolution fused with the [shortcut] behind
+ * it (fuse_shortcut=1) has no buffer of its own: its output is the shortcut's (the sum, activated). */
 int nbl_net_layer_output(nbl_net *net, int layer, float *host, size_t count);
+/* The max-pool argmax table the reference's forward keeps for its backward pass (pooling_layer.cc:132,140):
+ * flat offsets into the layer's input tensor.  Kept only when the [net] section says pool_index=1 (a key the
+ * reference ignores); inference never reads the table, so by default it is not written. */
 int nbl_net_pool_index(nbl_net *net, int layer, unsigned *host, size_t count);
+/* Convolutional layers: tile shape index and number of k slices (1 = unsplit) of the layer's most recent launch
+ * (nbl_conv2d_plan_last_launch), and a way to pin both (variant < 0: searched on first use; split: -1 searched,
+ * 0 never, 1 cost model, 2..8 that many slices) so that a run can be repeated with exactly the launches of another. */
+int nbl_net_conv_last_launch(nbl_net *net, int layer, int *variant, int *slices);
+int nbl_net_conv_pin_launch(nbl_net *net, int layer, int variant, int split);
 /* the softmax layer skips its device->host copy when enabled = 0 (throughput measurement) */
 int nbl_net_softmax_copy(nbl_net *net, int enabled);
 /* enabled = 1 (also the [net] key hip_graph=1, which the reference ignores): nbl_net_forward records the

@@ -168,8 +168,24 @@ int nbl_net_pool_index(nbl_net *n, int i, unsigned *host, size_t count) {
         layer_t *l = layer_at(n, i);
         if(l->layer_type != MAXPOOL_LAYER) throw std::runtime_error("Error: not a maxpool layer");
         if(count != (size_t)l->output_size * n->net->batch_size) throw std::runtime_error("Error: index buffer has the wrong size");
+        if(!static_cast<pooling_layer_t*>(l)->index_dev) throw std::runtime_error("Error: the argmax table is not kept (set pool_index=1 in [net])");
         nbl_check(n->net->ctx, nbl_d2h(n->net->ctx, host, static_cast<pooling_layer_t*>(l)->index_dev,
                                        count * sizeof(unsigned)), "nbl_d2h"));
+}
+
+int nbl_net_conv_last_launch(nbl_net *n, int i, int *variant, int *slices) {
+    NBL_NET_TRY(
+        layer_t *l = layer_at(n, i);
+        if(l->layer_type != CONVOLUTIONAL_LAYER) throw std::runtime_error("Error: not a convolutional layer");
+        static_cast<convolutional_layer_t*>(l)->last_launch(variant, slices));
+}
+
+int nbl_net_conv_pin_launch(nbl_net *n, int i, int variant, int split) {
+    NBL_NET_TRY(
+        layer_t *l = layer_at(n, i);
+        if(l->layer_type != CONVOLUTIONAL_LAYER) throw std::runtime_error("Error: not a convolutional layer");
+        n->net->invalidate_graph();
+        static_cast<convolutional_layer_t*>(l)->pin_launch(variant, split));
 }
 
 int nbl_net_softmax_copy(nbl_net *n, int enabled) {

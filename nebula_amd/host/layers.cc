@@ -187,6 +187,17 @@ void convolutional_layer_t::_forward_() {
               "nbl_conv2d_fwd");
 }
 
+void convolutional_layer_t::last_launch(int *variant, int *slices) const {
+    if(!plan) throw std::runtime_error("Error: convolutional layer has no weights (init_weight not called)");
+    nbl_check(network->ctx, nbl_conv2d_plan_last_launch(plan, variant, slices), "nbl_conv2d_plan_last_launch");
+}
+
+void convolutional_layer_t::pin_launch(int variant, int split) {
+    if(!plan) throw std::runtime_error("Error: convolutional layer has no weights (init_weight not called)");
+    nbl_check(network->ctx, nbl_conv2d_plan_set_variant(plan, variant), "nbl_conv2d_plan_set_variant");
+    nbl_check(network->ctx, nbl_conv2d_plan_set_split(plan, split), "nbl_conv2d_plan_set_split");
+}
+
 void convolutional_layer_t::weight_fields(std::vector<weight_field_t> &out) const {
     const unsigned fan_in = input_channel * filter_size * filter_size;
     out.push_back(weight_field_t{ WEIGHT_BIAS, num_filters, fan_in });
@@ -318,7 +329,7 @@ void pooling_layer_t::init(section_config_t m_section_config) {
     output_channel = input_channel;
     output_size    = output_height * output_width * output_channel;
     alloc_output();
-    if(layer_type == MAXPOOL_LAYER && network->ctx) {
+    if(layer_type == MAXPOOL_LAYER && network->ctx && network->pool_index) {
         const size_t bytes = sizeof(unsigned) * (size_t)output_size * network->batch_size;
         nbl_check(network->ctx, nbl_malloc(network->ctx, (void**)&index_dev, bytes), "nbl_malloc(index)");
         nbl_check(network->ctx, nbl_fill_zero(network->ctx, index_dev, bytes), "nbl_fill_zero(index)");

@@ -83,6 +83,11 @@ public:
     // pointer becomes an alias of that buffer.  Returns false (and changes nothing) when the pair cannot
     // be fused (up-sampling shortcut, or a shortcut whose source is this very layer).
     bool fuse_with(class shortcut_layer_t *m_shortcut);
+    // Tile shape and k-split of the kernel: what the most recent forward used, and a way to pin both
+    // (variant < 0: searched on first use; split as nbl_conv2d_plan_set_split).
+    void last_launch(int *variant, int *slices) const;
+    void pin_launch(int variant, int split);
+    bool is_fused() const { return fused_shortcut != NULL; }
 private:
     void pack();
     bool batch_normalize;
@@ -123,7 +128,7 @@ public:
     void init_weight() {}
     void store_weight(std::fstream &) {}
     void _forward_();
-    unsigned *index_dev;       // maxpool argmax: flat offsets into the input tensor
+    unsigned *index_dev;       // maxpool argmax: flat offsets into the input tensor (NULL unless [net] pool_index=1)
 };
 
 // models/layers/shortcut_layer.h

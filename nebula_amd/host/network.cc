@@ -24,7 +24,7 @@ network_t::network_t() :
     run_type(UNDEFINED_RUN), num_threads(1),
     learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
     input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
-    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1), defer_host_copy(false),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1), pool_index(false), defer_host_copy(false),
     input_layer(NULL), output_layer(NULL), num_layers(0) {}
 
 network_t::~network_t() {}
@@ -126,6 +126,7 @@ void inference_net_t::build(config_t &config) {
             sc.get_setting("batch", &batch_size);
             sc.get_setting("fuse_shortcut", &fuse_shortcut);
             sc.get_setting("hip_graph", &use_graph);
+            sc.get_setting("pool_index", &pool_index);
             if(sc.exists("conv_split")) { unsigned v = 0; sc.get_setting("conv_split", &v); conv_split = v ? 1 : 0; }
             if(batch_override) batch_size = batch_override;
             input_size = input_height * input_width * input_channel;
@@ -161,8 +162,19 @@ void inference_net_t::build(config_t &config) {
     if(!output_layer && !layers.empty()) output_layer = layers.back();
     if(fuse_shortcut)
         for(unsigned i = 1; i < num_layers; i++)
-            if(layers[i]->layer_type == SHORTCUT_LAYER && layers[i - 1]->layer_type == CONVOLUTIONAL_LAYER)
-                static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
+            if(layers[i]->layer_type == SHORTCUT_LAYER && layers[i - 1]->layer_type == CONVOLUTIONAL_LAYER) {
+                // A fused convolution never writes its own (pre-add) output.  That is only safe when nothing but the
+                // shortcut behind it reads that output: a later shortcut whose `hops` land on this convolution (or
+                // on an alias of it) needs the pre-add tensor, so the pair stays unfused.
+                bool read_elsewhere = false;
+                for(unsigned j = i + 1; j < num_layers && !read_elsewhere; j++)
+                    if(layers[j]->layer_type == SHORTCUT_LAYER) {
+                        const layer_t *conn = static_cast<shortcut_layer_t*>(layers[j])->connection;
+                        read_elsewhere = conn == layers[i - 1] || (conn && conn->output_data_dev == layers[i - 1]->output_data_dev);
+                    }
+                if(!read_elsewhere)
+                    static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
+            }
     for(unsigned i = 0; i < num_layers; i++)
         if(layers[i]->layer_type == LSTM_LAYER || layers[i]->layer_type == RNN_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
 }
@@ -255,23 +267,26 @@ void inference_net_t::run(const std::string) {
     nbl_check(ctx, nbl_sync(ctx), "nbl_sync");
 }
 
-// Layer i, with the rows narrowed to the final time step from the first layer after the last LSTM on
-// when last_step_only is set: that layer reads the last B rows of its producer, everything after it
-// works on B rows.  The pointer and the row count are restored right after the call.
+// Layer i, with the rows narrowed to the final time step behind the last recurrent layer when last_step_only is
+// set.  A layer there that reads the recurrent layer's T*B rows -- directly, or through layers that only alias
+// their producer's buffer (dropout, cost) -- is pointed at the last B rows for the duration of its call; every
+// layer behind the recurrent layer works on B rows.  Pointer and row count are restored right after the call.
 void inference_net_t::run_layer(unsigned i) {
     const bool narrow = last_step_only && is_recurrent && time_step > 1 && first_after_lstm >= 0 &&
                         (int)i >= first_after_lstm;
     if(!narrow) { layers[i]->_forward_(); return; }
     const unsigned rows = batch_size, seqs = batch_size / time_step;
-    layer_t *producer = layers[i]->prev_layer;
-    float *saved = producer ? producer->output_data_dev : NULL;
-    if((int)i == first_after_lstm && producer)
-        producer->output_data_dev += (size_t)(time_step - 1) * seqs * producer->output_size;
+    layer_t *src = layers[i]->prev_layer;       // the layer whose output pointer layer i reads
+    const layer_t *real = src;                  // ... and the layer that wrote the rows behind that pointer
+    while(real && (real->layer_type == DROPOUT_LAYER || real->layer_type == COST_LAYER)) real = real->prev_layer;
+    const bool reads_all_steps = real != NULL && real == layers[first_after_lstm - 1];
+    float *saved = src ? src->output_data_dev : NULL;
+    if(reads_all_steps) src->output_data_dev += (size_t)(time_step - 1) * seqs * src->output_size;
     batch_size = seqs;
     try { layers[i]->_forward_(); }
-    catch(...) { batch_size = rows; if(producer) producer->output_data_dev = saved; throw; }
+    catch(...) { batch_size = rows; if(src) src->output_data_dev = saved; throw; }
     batch_size = rows;
-    if(producer) producer->output_data_dev = saved;
+    if(src) src->output_data_dev = saved;
 }
 
 void inference_net_t::forward_eager() {

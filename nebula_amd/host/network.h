@@ -54,6 +54,10 @@ public:
     // the patch rows between blocks, 1 = wherever the cost model says so; absent = measured per layer on
     // first use.  With 0 a convolution's result does not depend on the tile shape the search picks.
     int conv_split;
+    // [net] key `pool_index=1` (a key the reference ignores): max-pooling layers also store the argmax table the
+    // reference's forward writes for its backward pass (models/layers/pooling_layer.cc:132,140).  Inference never
+    // reads it, so by default it is neither allocated nor written (a third of a max-pool's memory traffic).
+    bool pool_index;
     // Set while inference_net_t::forward() records or replays a HIP graph: a layer that copies to the host queues
     // the copy on the stream instead of waiting for it, and forward() waits once at its end.
     bool defer_host_copy;

@@ -35,6 +35,8 @@ SIGNATURES = {
     "nbl_net_forward_timed": (C.c_int, [_vp, C.POINTER(C.c_float)]),
     "nbl_net_layer_output": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
     "nbl_net_pool_index": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
+    "nbl_net_conv_last_launch": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "nbl_net_conv_pin_launch": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int]),
     "nbl_net_softmax_copy": (C.c_int, [_vp, C.c_int]),
     "nbl_net_set_graph": (C.c_int, [_vp, C.c_int]),
     "nbl_net_graph_active": (C.c_int, [_vp]),
@@ -178,6 +180,16 @@ class Network:
         out = np.empty(info["output_size"] * self.batch_size, np.uint32)
         self._check(lib().nbl_net_pool_index(self.h, i, out.ctypes.data, out.size))
         return out
+
+    def conv_last_launch(self, i):
+        """(tile shape index, k slices) of convolutional layer i's most recent launch."""
+        v, g = C.c_int(), C.c_int()
+        self._check(lib().nbl_net_conv_last_launch(self.h, i, C.byref(v), C.byref(g)))
+        return v.value, g.value
+
+    def conv_pin_launch(self, i, variant, split):
+        """Pin layer i's tile shape (variant < 0: searched) and k-split (-1 searched, 0 never, 1 cost model, 2..8 slices)."""
+        self._check(lib().nbl_net_conv_pin_launch(self.h, i, variant, split))
 
     def softmax_copy(self, enabled):
         lib().nbl_net_softmax_copy(self.h, 1 if enabled else 0)

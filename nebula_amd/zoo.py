@@ -27,9 +27,11 @@ def _fc(output, activation):
 _TAIL = "\n[softmax]\ngroups=1\n\n[cost]\ntype=l2\n"
 
 
-def conv1_pool_cfg(batch=32):
-    """AlexNet conv1 + ReLU + 3x3/s2 maxpool."""
-    return _net(batch, 227, 227, 3) + _conv(96, 11, 4, 0, "relu") + _pool("maxpool", 3, 2, 0)
+def conv1_pool_cfg(batch=32, pool_index=False):
+    """AlexNet conv1 + ReLU + 3x3/s2 maxpool.  pool_index: also keep the argmax table the reference's forward
+    writes for its backward pass (a [net] key the reference ignores)."""
+    return (_net(batch, 227, 227, 3, "pool_index=1\n" if pool_index else "") + _conv(96, 11, 4, 0, "relu")
+            + _pool("maxpool", 3, 2, 0))
 
 
 def alexnet_cfg(batch=128):

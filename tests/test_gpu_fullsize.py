@@ -38,7 +38,7 @@ def oracle_forward(cfg, blob, x):
 
 def test_config1_conv1_relu_maxpool_full_size():
     print("CASE config 1 full size", flush=True)
-    cfg = zoo.conv1_pool_cfg(32)
+    cfg = zoo.conv1_pool_cfg(32, pool_index=True)
     rng = np.random.default_rng(1)
     x = rng.random((32, 3, 227, 227), dtype=np.float32)
     net, blob = build(cfg)

@@ -49,7 +49,7 @@ def test_golden_network(golden_dir, name):
 def test_maxpool_index_through_layer(golden_dir):
     # identical input to the pooling layer -> identical argmax table: feed the pool layer directly
     from nebula_amd.net import Network
-    cfg = "[net]\nbatch=2\nheight=13\nwidth=11\nchannels=3\n[maxpool]\nsize=3\nstride=2\n"
+    cfg = "[net]\nbatch=2\nheight=13\nwidth=11\nchannels=3\npool_index=1\n[maxpool]\nsize=3\nstride=2\n"
     rng = np.random.default_rng(3)
     x = rng.standard_normal((2, 3, 13, 11)).astype(np.float32)
     with Network(cfg) as net:
@@ -58,6 +58,14 @@ def test_maxpool_index_through_layer(golden_dir):
         wy, widx = ob.maxpool_forward(x, 3, 2, 1)
         np.testing.assert_array_equal(net.output(0).view(np.uint32), wy.ravel().view(np.uint32))
         np.testing.assert_array_equal(net.pool_index(0), widx.ravel())
+    # without the key the values are the same and the table is not kept
+    from nebula_amd.net import NetworkError
+    with Network(cfg.replace("pool_index=1\n", "")) as net:
+        net.set_input(x)
+        net.forward()
+        np.testing.assert_array_equal(net.output(0).view(np.uint32), wy.ravel().view(np.uint32))
+        with pytest.raises(NetworkError, match="pool_index=1"):
+            net.pool_index(0)
 
 
 def test_cfg_errors_are_reported():

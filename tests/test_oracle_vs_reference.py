@@ -1,12 +1,16 @@
 """The CPU oracle against the compiled, unmodified reference (oracle/_ref/libnebula_ref.so) on
 seeded random inputs.  That library can only be built where the reference tree exists, so these
 tests skip elsewhere (the committed golden vectors cover the same ground there)."""
+import os
+
 import numpy as np
 import pytest
 
 from oracle import binding as ob
 
-pytestmark = pytest.mark.skipif(ob.ref() is None, reason="reference tree not present")
+# decided from the tree alone: nothing is compiled or loaded while pytest collects, and nothing at all where the
+# reference is absent
+pytestmark = pytest.mark.skipif(not os.path.isdir(ob.REFERENCE_ROOT), reason="reference tree not present")
 
 
 def bits(a):
