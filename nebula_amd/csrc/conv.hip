@@ -164,9 +164,22 @@ void conv_igemm_kernel(const ConvArgs a) {
     constexpr int A_VEC = BK * BM / 4;                 // float4s in a weight tile
     constexpr int RA = (A_VEC + NTHREADS - 1) / NTHREADS;
     static_assert(RA <= 2, "weight tile needs at most two float4 per thread");
+    // LDS layout of a k-tile.  The table-driven gathers give a thread RB consecutive patch rows of ONE pixel, so their
+    // tiles are kept as quads of k: [k / 4][column][k % 4] -- a thread's four rows are one 16-byte LDS write (four
+    // 4-byte writes cost the matrix pipe about 4 % in a stand-alone copy of this loop), and a lane fetches its operands
+    // of four k-steps with one 16-byte read.  Lanes 0-31 then feed the k of the even quads and lanes 32-63 the k of the
+    // odd quads to the MFMAs; any pairing of k is legal as long as both operands use the same one, and the packed
+    // weights are laid out to match ([Kp / 4][Mp][4]).  The 1x1 gather loads four PIXELS of one row per thread and
+    // keeps k-major rows ([k][column], rows k and k+1 in different bank halves through the +32).
+    constexpr bool KQ = !VEC4;
+    constexpr int PADQ = 8;                            // quad layout: row pitch (BM + 8) * 16 bytes puts consecutive quads half the banks apart
+    static_assert(VEC4 || RB % 4 == 0, "a thread's patch rows must be whole quads");
 
-    __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
+    __shared__ __attribute__((aligned(16))) float As[KQ ? 2 * (BK / 4) * (BM + PADQ) * 4 : 2 * BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[KQ ? 2 * (BK / 4) * (BN + PADQ) * 4 : 2 * BK * LDB];
+    constexpr int A_BUF = KQ ? (BK / 4) * (BM + PADQ) * 4 : BK * LDA;      // floats per buffer
+    constexpr int B_BUF = KQ ? (BK / 4) * (BN + PADQ) * 4 : BK * LDB;
+    constexpr int A_QROW = (BM + PADQ) * 4, B_QROW = (BN + PADQ) * 4;       // floats between quads (quad layout)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
@@ -229,10 +242,14 @@ void conv_igemm_kernel(const ConvArgs a) {
         for(int r = 0; r < RB; r++) vec_off[r] = (unsigned)(px.xbase + (krow0 + r * KGROUPS) * a.OHW) * 4u;
     }
     const __amdgpu_buffer_rsrc_t wres = make_rsrc(a.wp, (unsigned)a.Kp * (unsigned)a.Mp * 4u);
+    // weight tile: k-major rows [16][BM] read as float4s along the filters, or quads [4][BM][4] read as one float4 per
+    // (quad, filter); either way a thread's piece sits at a constant offset from the k-tile's start
     const unsigned w_off0 = A_VEC >= NTHREADS || tid < A_VEC
-        ? (unsigned)((tid / (BM / 4)) * a.Mp + (tid % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
+        ? (KQ ? (unsigned)((tid / BM) * a.Mp + tid % BM + ld_m0) * 16u
+              : (unsigned)((tid / (BM / 4)) * a.Mp + (tid % (BM / 4)) * 4 + ld_m0) * 4u) : OOB_OFFSET;
     const unsigned w_off1 = RA > 1 && (A_VEC >= 2 * NTHREADS || tid + NTHREADS < A_VEC)
-        ? (unsigned)(((tid + NTHREADS) / (BM / 4)) * a.Mp + ((tid + NTHREADS) % (BM / 4)) * 4 + ld_m0) * 4u : OOB_OFFSET;
+        ? (KQ ? (unsigned)(((tid + NTHREADS) / BM) * a.Mp + (tid + NTHREADS) % BM + ld_m0) * 16u
+              : (unsigned)(((tid + NTHREADS) / (BM / 4)) * a.Mp + ((tid + NTHREADS) % (BM / 4)) * 4 + ld_m0) * 4u) : OOB_OFFSET;
     // tap-major: bit i*ksize+j is set when that tap of this thread's pixel is OUTSIDE the image; bit 31 is always
     // set and stands for the padding k-tiles behind the last patch row
     unsigned outmask = 0x80000000u;
@@ -301,19 +318,19 @@ void conv_igemm_kernel(const ConvArgs a) {
     auto store_tile = [&](const Stage &st, int buf) {
         if(VEC4) {
             #pragma unroll
-            for(int r = 0; r < RB; r++) *reinterpret_cast<vec4f*>(&Bs[buf][krow0 + r * KGROUPS][ncol * 4]) = st.b4[r];
+            for(int r = 0; r < RB; r++) *reinterpret_cast<vec4f*>(&Bs[buf * B_BUF + (krow0 + r * KGROUPS) * LDB + ncol * 4]) = st.b4[r];
         } else {
             #pragma unroll
-            for(int r = 0; r < RB; r++) Bs[buf][krow0 + r][ncol] = st.b[r];
+            for(int q = 0; q < RB / 4; q++)
+                *reinterpret_cast<vec4f*>(&Bs[buf * B_BUF + (krow0 / 4 + q) * B_QROW + ncol * 4]) =
+                    vec4f{st.b[4 * q], st.b[4 * q + 1], st.b[4 * q + 2], st.b[4 * q + 3]};
         }
-        {
-            const int row = tid / (BM / 4), col4 = tid % (BM / 4);
-            if(A_VEC >= NTHREADS || tid < A_VEC) *reinterpret_cast<vec4f*>(&As[buf][row][col4 * 4]) = st.a0;
-        }
-        if(RA > 1) {
-            const int v = tid + NTHREADS;
-            const int row = v / (BM / 4), col4 = v % (BM / 4);
-            if(A_VEC >= 2 * NTHREADS || v < A_VEC) *reinterpret_cast<vec4f*>(&As[buf][row][col4 * 4]) = st.a1;
+        #pragma unroll
+        for(int u = 0; u < RA; u++) {
+            const int v = tid + u * NTHREADS;
+            float *dst = KQ ? &As[buf * A_BUF + (v / BM) * A_QROW + (v % BM) * 4]
+                            : &As[buf * A_BUF + (v / (BM / 4)) * LDA + (v % (BM / 4)) * 4];
+            if(A_VEC >= (u + 1) * NTHREADS || v < A_VEC) *reinterpret_cast<vec4f*>(dst) = u == 0 ? st.a0 : st.a1;
         }
     };
 
@@ -321,36 +338,69 @@ void conv_igemm_kernel(const ConvArgs a) {
 
     // Rows and columns are dealt to the MFMA tiles of a wave interleaved: tile i of the wave holds rows
     // l*MT + i (l = 0..31) and tile j holds columns l*NT + j.  A lane therefore finds the MT (NT)
-    // operand values of one k in adjacent LDS words and fetches them with one wide read at a
-    // compile-time offset, and in the epilogue it owns NT adjacent pixels of each of its rows.
-    const float *a_lane = &As[0][half][wm * MT * 32 + l32 * MT];
-    const float *b_lane = &Bs[0][half][wn * NT * 32 + l32 * NT];
-    // all MFMAs of one resident k-tile; the operands of k-step ks+1 are fetched from LDS before the
-    // MFMAs of k-step ks are issued
-    auto compute_tile = [&](int buf) {
-        const float *ap = a_lane + buf * (BK * LDA), *bp = b_lane + buf * (BK * LDB);
-        float av[2][MT], bv[2][NT];
-        #pragma unroll
-        for(int i = 0; i < MT; i++) av[0][i] = ap[i];
-        #pragma unroll
-        for(int j = 0; j < NT; j++) bv[0][j] = bp[j];
-        #pragma unroll
-        for(int ks = 0; ks < BK / 2; ks++) {
-            const int cur = ks & 1, nxt = cur ^ 1;
-            if(ks + 1 < BK / 2) {           // operands of the next k-step, in flight behind this step's MFMAs
+    // operand values of one k in adjacent LDS words, and in the epilogue it owns NT adjacent pixels of each of its rows.
+    //
+    // ALL operands of a k-tile are fetched into registers (8 k-steps x (MT + NT) values): once every wave holds
+    // its copy, the tile's LDS buffer is free, so the one barrier per k-tile can sit in the MIDDLE of the tile's
+    // MFMAs instead of at their end -- the operands of the next tile are then read from LDS behind the second half of
+    // this tile's MFMAs, and no wave starts a tile by waiting for LDS.  (In a stand-alone copy of this loop, 64x64
+    // tile, 6 blocks per CU: 81 % of the matrix peak with the barrier at the end of the tile, 88-89 % here.)
+    // Operand registers: quad layout -- opa[h][i] holds k-steps 4h..4h+3 of row tile i; k-major layout -- element j
+    // of opa[h][i] is k-step 4h + j all the same, fetched with 4-byte reads.
+    struct Operands { vec4f a[2][MT]; vec4f b[2][NT]; };
+    const int a_lane = KQ ? half * A_QROW + (wm * MT * 32 + l32 * MT) * 4 : half * LDA + wm * MT * 32 + l32 * MT;
+    const int b_lane = KQ ? half * B_QROW + (wn * NT * 32 + l32 * NT) * 4 : half * LDB + wn * NT * 32 + l32 * NT;
+    // the operands of k-steps 4h..4h+3 of the tile in LDS buffer `buf`
+    auto read_half = [&](int buf, int h, vec4f (&oa)[MT], vec4f (&ob)[NT]) {
+        if(KQ) {
+            const float *ap = &As[buf * A_BUF + a_lane + 2 * h * A_QROW], *bp = &Bs[buf * B_BUF + b_lane + 2 * h * B_QROW];
+            #pragma unroll
+            for(int i = 0; i < MT; i++) oa[i] = *reinterpret_cast<const vec4f*>(ap + 4 * i);
+            #pragma unroll
+            for(int j = 0; j < NT; j++) ob[j] = *reinterpret_cast<const vec4f*>(bp + 4 * j);
+        } else {
+            const float *ap = &As[buf * A_BUF + a_lane + 8 * h * LDA], *bp = &Bs[buf * B_BUF + b_lane + 8 * h * LDB];
+            #pragma unroll
+            for(int e = 0; e < 4; e++) {
                 #pragma unroll
-                for(int i = 0; i < MT; i++) av[nxt][i] = ap[(ks + 1) * 2 * LDA + i];
+                for(int i = 0; i < MT; i++) oa[i][e] = ap[e * 2 * LDA + i];
                 #pragma unroll
-                for(int j = 0; j < NT; j++) bv[nxt][j] = bp[(ks + 1) * 2 * LDB + j];
+                for(int j = 0; j < NT; j++) ob[j][e] = bp[e * 2 * LDB + j];
             }
-            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // MFMAs of k-steps [s0, s1) of the tile whose operands are in `o`
+    auto mfma_steps = [&](const Operands &o, auto s0_, auto s1_) {
+        constexpr int s0 = decltype(s0_)::value, s1 = decltype(s1_)::value;
+        #pragma unroll
+        for(int ks = s0; ks < s1; ks++)
             #pragma unroll
             for(int i = 0; i < MT; i++)
                 #pragma unroll
                 for(int j = 0; j < NT; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cur][i], bv[cur][j], acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.a[ks / 4][i][ks % 4], o.b[ks / 4][j][ks % 4], acc[i][j], 0, 0, 0);
+    };
+    constexpr int KS_BEFORE = MT * NT >= 2 ? 1 : 2;       // k-steps multiplied before the barrier
+    typedef std::integral_constant<int, 0> ks_first;
+    typedef std::integral_constant<int, KS_BEFORE> ks_split;
+    typedef std::integral_constant<int, BK / 2> ks_last;
+    Operands cur;
+    // One k-tile: `cur` holds its operands; `st` holds the next k-tile, which goes to LDS buffer `buf`.
+    auto tile_step = [&](const Stage &st, int buf) {
+        mfma_steps(cur, ks_first(), ks_split());
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(st, buf);
+        __syncthreads();
+        vec4f na[MT], nb[NT];
+        read_half(buf, 0, na, nb);                  // next tile's first half, in flight behind the MFMAs below
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_steps(cur, ks_split(), ks_last());
+        __builtin_amdgcn_sched_barrier(0);
+        #pragma unroll
+        for(int i = 0; i < MT; i++) cur.a[0][i] = na[i];
+        #pragma unroll
+        for(int j = 0; j < NT; j++) cur.b[0][j] = nb[j];
+        read_half(buf, 1, cur.a[1], cur.b[1]);      // needed four k-steps into the next tile
     };
 
     // Short epilogue of a full tile whose rows are reached as base pointer + 32-bit byte offset: per row
@@ -606,32 +656,28 @@ void conv_igemm_kernel(const ConvArgs a) {
     load_ktab(kt_begin);
     ld_next(st0);
     ld_next(st1);
-    store_tile(st0, 0);
-    __syncthreads();
-
     #pragma unroll
     for(int i = 0; i < MT; i++)
         #pragma unroll
         for(int j = 0; j < NT; j++)
             #pragma unroll
             for(int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    store_tile(st0, 0);
+    __syncthreads();
+    read_half(0, 0, cur.a[0], cur.b[0]);
+    read_half(0, 1, cur.a[1], cur.b[1]);
+
     for(int kt = kt_begin; kt < kt_end - 2; kt += 2) {
-        // k-tile kt is in LDS buffer 0, kt+1 is in flight in stage 1
+        // operands of k-tile kt are in registers, kt+1 is in flight in stage 1
         ld_next(st0);
-        compute_tile(0);
-        store_tile(st1, 1);
-        __syncthreads();
-        // k-tile kt+1 is in LDS buffer 1, kt+2 is in flight in stage 0
+        tile_step(st1, 1);
+        // operands of k-tile kt+1 are in registers, kt+2 is in flight in stage 0
         ld_next(st1);
-        compute_tile(1);
-        store_tile(st0, 0);
-        __syncthreads();
+        tile_step(st0, 0);
     }
     // last pair: nothing left to load
-    compute_tile(0);
-    store_tile(st1, 1);
-    __syncthreads();
-    compute_tile(1);
+    tile_step(st1, 1);
+    mfma_steps(cur, ks_first(), ks_last());
     if(split_block) store_partial();
     else epilogue(tile);
 }
@@ -761,7 +807,9 @@ constexpr int NUM_VARIANTS = sizeof(VARIANTS) / sizeof(VARIANTS[0]);
 struct nbl_conv_plan {
     unsigned C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp;
     int act; bool has_scale;
-    float *wp_dev; int2 *ktab_dev; float *g_dev; float *b_dev;
+    float *wp_dev;      // packed weights as quads of patch rows, [Kp / 4][Mp][4] (every gather but the 1x1 vector gather)
+    float *wp_rows_dev; // the same as k-major rows [Kp][Mp], kept only for layers the 1x1 vector gather can take
+    int2 *ktab_dev; float *g_dev; float *b_dev;
     bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 31)
     int variant;   // < 0: chosen per call
     unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
@@ -857,16 +905,20 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
     p->split_mode = -1; p->tuned_slices = 0; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
-    p->wp_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
+    p->wp_dev = NULL; p->wp_rows_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
     p->tap_major = ksize > 1 && ksize * ksize <= 31 && C % CONV_BK == 0;
 
-    // [F][K] -> [Kp][Mp], zero padded
-    std::vector<float> wp((size_t)p->Kp * p->Mp, 0.0f);
+    // [F][K] -> quads of patch rows [Kp / 4][Mp][4], zero padded; layers the 1x1 vector gather can take (decided per
+    // call: it also needs a 16-byte aligned input) keep k-major rows [Kp][Mp] as well
+    const bool vec4_geometry = ksize == 1 && stride == 1 && pad == 0 && (p->OH * p->OW) % 4 == 0 && p->K == p->Kp;
+    std::vector<float> wp((size_t)p->Kp * p->Mp, 0.0f), wrows(vec4_geometry ? (size_t)p->Kp * p->Mp : 0, 0.0f);
     const unsigned taps = ksize * ksize;
     for(unsigned f = 0; f < F; f++)
         for(unsigned kk = 0; kk < p->K; kk++) {
             const unsigned row = patch_row(kk / taps, kk % taps, taps, p->tap_major);    // kk = c*taps + t in the file
-            wp[(size_t)row * p->Mp + f] = weight_host[(size_t)f * p->K + kk];
+            const float v = weight_host[(size_t)f * p->K + kk];
+            wp[((size_t)(row / 4) * p->Mp + f) * 4 + row % 4] = v;
+            if(vec4_geometry) wrows[(size_t)row * p->Mp + f] = v;
         }
     std::vector<float> g(p->Mp, 0.0f), b(p->Mp, 0.0f);
     nbl_fold_batchnorm(bias_host, scale_host, mean_host, var_host, F, g.data(), b.data());
@@ -881,6 +933,8 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
        (rc = nbl_malloc(ctx, (void**)&p->g_dev, g.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_malloc(ctx, (void**)&p->b_dev, b.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_h2d(ctx, p->wp_dev, wp.data(), wp.size() * sizeof(float))) != NBL_OK ||
+       (vec4_geometry && ((rc = nbl_malloc(ctx, (void**)&p->wp_rows_dev, wrows.size() * sizeof(float))) != NBL_OK ||
+                          (rc = nbl_h2d(ctx, p->wp_rows_dev, wrows.data(), wrows.size() * sizeof(float))) != NBL_OK)) ||
        (rc = nbl_h2d(ctx, p->ktab_dev, tab.data(), tab.size() * sizeof(int2))) != NBL_OK ||
        (rc = nbl_h2d(ctx, p->g_dev, g.data(), g.size() * sizeof(float))) != NBL_OK ||
        (rc = nbl_h2d(ctx, p->b_dev, b.data(), b.size() * sizeof(float))) != NBL_OK) {
@@ -894,7 +948,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
 int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->ttab_dev);
-    nbl_free(ctx, p->wp_dev); nbl_free(ctx, p->ktab_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev);
+    nbl_free(ctx, p->wp_dev); nbl_free(ctx, p->wp_rows_dev); nbl_free(ctx, p->ktab_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev);
     nbl_free(ctx, p->ws_dev);
     delete p;
     return NBL_OK;
@@ -974,8 +1028,7 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     a.ttab = p->ttab_dev; a.ksize = (int)p->k; a.plane_bytes = p->H * p->W * 4u;
     int gather = p->pad == 0 ? GATHER_NOPAD : GATHER_PADDED;
     if(p->tap_major) gather = GATHER_TAP_MAJOR;
-    if(p->k == 1 && p->stride == 1 && p->pad == 0 && (p->OH * p->OW) % 4 == 0 && ((size_t)x_dev & 15) == 0 && p->K == p->Kp)
-        gather = GATHER_1X1_VEC4;
+    if(p->wp_rows_dev && ((size_t)x_dev & 15) == 0) { gather = GATHER_1X1_VEC4; a.wp = p->wp_rows_dev; }
     a.whole_tiles = (int)blocks; a.split = 1; a.n_start = 0; a.n_tail = 0; a.ws = NULL;
     size_t grid = blocks;
     if(slices && p->F <= 65535) {     // the finishing kernel's grid has one row per filter
