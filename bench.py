@@ -181,6 +181,112 @@ def image_input(args):
     ctx.close()
 
 
+def memory_bound_kernels(args):
+    """The bandwidth-bound kernels at the sizes the BASELINE networks give them, each timed on its own through the C ABI
+    (HIP events on the library's stream, back-to-back launches).  For every kernel: algorithmic bytes per launch (the
+    tensors it must read and write once), microseconds per launch and the fraction of the 8 TB/s HBM peak.  The copy
+    kernel is the yardstick: what a plain read-once / write-once stream reaches on this machine."""
+    from nebula_amd import hip
+    ctx = hip.Ctx(0)
+    l = hip.lib()
+    rng = np.random.default_rng(3)
+    out = []
+
+    def timed(name, nbytes, launch, note=""):
+        for _ in range(args.warmup):
+            launch()
+        ctx.sync()
+        ctx.timer_start()
+        for _ in range(args.steps):
+            launch()
+        us = ctx.timer_stop() * 1e3 / args.steps
+        gbs = nbytes / us / 1e3
+        rec = {"kernel": name, "bytes": int(nbytes), "us": round(us, 2), "GBps": round(gbs, 1), "frac_of_8TBps": round(gbs / PEAK_HBM_GBS, 3)}
+        if note:
+            rec["note"] = note
+        out.append(rec)
+        log(rec)
+
+    def rand(shape):
+        # device-resident random data without a 200 MB host array per tensor: one 16 MB block repeated
+        n = int(np.prod(shape))
+        block = rng.standard_normal(min(n, 1 << 22)).astype(np.float32)
+        a = ctx.empty(shape)
+        reps = -(-n // block.size)
+        host = np.tile(block, reps)[:n]
+        a.upload(host)
+        return a
+
+    # yardstick
+    n = 64 << 20
+    src, dst = rand((n,)), ctx.empty((n,))
+    timed("copy (nbl_copy_d2d) 256 MiB", 2 * 4 * n, lambda: ctx.copy(dst, src))
+    src.free(); dst.free()
+
+    # max-pool 3x3 / 2 on ResNet-50's stem output at batch 64, as inference runs it (no argmax table) and as the
+    # reference's forward does (table written)
+    B, C_, H = 64, 64, 112
+    x = rand((B, C_, H, H)); y = ctx.empty((B, C_, 56, 56)); idx = ctx.empty((B, C_, 56, 56), dtype=np.uint32)
+    io = 4 * (x.size + y.size)
+    timed("maxpool 3x3/2 64x64x112x112 (no argmax table)", io,
+          lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, None, B, C_, H, H, 3, 2, 0, hip.POOL_MAX)))
+    timed("maxpool 3x3/2 64x64x112x112 (+ argmax table)", io + 4 * y.size,
+          lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, idx.ptr, B, C_, H, H, 3, 2, 0, hip.POOL_MAX)))
+    x.free(); y.free(); idx.free()
+    # VGG-16's first max-pool 2x2 / 2 at batch 32
+    x = rand((32, 64, 224, 224)); y = ctx.empty((32, 64, 112, 112))
+    timed("maxpool 2x2/2 32x64x224x224 (no argmax table)", 4 * (x.size + y.size),
+          lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, None, 32, 64, 224, 224, 2, 2, 0, hip.POOL_MAX)))
+    x.free(); y.free()
+    # ResNet-50's closing 7x7 average pool
+    x = rand((64, 2048, 7, 7)); y = ctx.empty((64, 2048))
+    timed("avgpool 7x7 64x2048x7x7", 4 * (x.size + y.size),
+          lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, None, 64, 2048, 7, 7, 7, 7, 0, hip.POOL_AVG)))
+    x.free(); y.free()
+
+    # shortcuts as stand-alone layers (fuse_shortcut=0): same shape, and a stage entry (stride 2, fewer channels)
+    prev = rand((64, 256, 56, 56)); conn = rand((64, 256, 56, 56)); y = ctx.empty((64, 256, 56, 56))
+    timed("shortcut same shape 64x256x56x56 + relu", 12 * y.size,
+          lambda: ctx.check(l.nbl_shortcut_fwd(ctx.h, prev.ptr, conn.ptr, y.ptr, 64, 256, 56, 56, 256, 56, 56, hip.ACT["relu"])))
+    # in-place activation, bias and batchnorm primitives on the same tensor
+    timed("activation relu in place, 51.4 M elements", 8 * y.size,
+          lambda: ctx.check(l.nbl_activation_fwd(ctx.h, y.ptr, y.size, hip.ACT["relu"])))
+    timed("activation leaky in place, 51.4 M elements", 8 * y.size,
+          lambda: ctx.check(l.nbl_activation_fwd(ctx.h, y.ptr, y.size, hip.ACT["leaky"])))
+    bias = rand((256,)); var = ctx.array(rng.uniform(0.5, 1.5, 256).astype(np.float32))
+    timed("forward_bias 64x256x56x56", 8 * y.size,
+          lambda: ctx.check(l.nbl_forward_bias(ctx.h, y.ptr, bias.ptr, 256, 56 * 56, 64)))
+    timed("batchnorm_inference 64x256x56x56", 8 * y.size,
+          lambda: ctx.check(l.nbl_batchnorm_inference(ctx.h, y.ptr, bias.ptr, var.ptr, bias.ptr, 256, 56 * 56, 64)))
+    prev.free(); y.free()
+    prev = rand((64, 512, 28, 28)); y = ctx.empty((64, 512, 28, 28))
+    timed("shortcut stage entry 64x256x56x56 -> 64x512x28x28 + relu", 8 * y.size + 4 * (64 * 256 * 28 * 28),
+          lambda: ctx.check(l.nbl_shortcut_fwd(ctx.h, prev.ptr, conn.ptr, y.ptr, 64, 256, 56, 56, 512, 28, 28, hip.ACT["relu"])),
+          note="residual counted as the 28x28 samples it adds; it touches every other 32-byte piece of two rows out of four")
+    prev.free(); conn.free(); y.free()
+
+    # softmax: the recurrent driver's 4096 x 10000 (all time steps), and 64 x 1000 / 128 x 1000 (image nets)
+    for rows, n_ in ((4096, 10000), (64, 10000), (64, 1000), (128, 1000)):
+        x = rand((rows, n_)); y = ctx.empty((rows, n_))
+        timed("softmax %d x %d" % (rows, n_), 8 * rows * n_,
+              lambda: ctx.check(l.nbl_softmax_fwd(ctx.h, x.ptr, y.ptr, rows, n_)))
+        x.free(); y.free()
+
+    # weight-streaming connected layers (the whole layer: product, split-K reduction, bias, relu)
+    for name, B_, I, O in (("VGG-16 fc6", 32, 25088, 4096), ("AlexNet fc6", 128, 9216, 4096), ("VGG-16 fc7", 32, 4096, 4096),
+                           ("LSTM projection (last step)", 64, 1024, 10000)):
+        w = (rng.standard_normal((O, 8)).astype(np.float32) * 0.01).repeat(I // 8, axis=1)
+        plan = ctx.fc_pack(w, np.zeros(O, np.float32), None, "relu")
+        del w
+        x = rand((B_, I)); y = ctx.empty((B_, O))
+        timed("connected %s  %d x %d -> %d" % (name, B_, I, O), 4 * (I * O + B_ * I + B_ * O), lambda: plan(x, out=y))
+        x.free(); y.free()
+    ctx.close()
+    worst = min(r["frac_of_8TBps"] for r in out[1:])
+    print(json.dumps({"metric": "memory-bound kernels, fraction of the 8 TB/s HBM peak (lowest of the kernels listed)", "value": worst,
+                      "unit": "fraction", "steps": args.steps, "warmup": args.warmup, "peak_GBps": PEAK_HBM_GBS, "kernels": out}), flush=True)
+
+
 def recurrent_driver(args):
     """The recurrent driver's test step (models/networks/recurrent.cc): one-hot words of a 10000-word vocabulary,
     T = 64 steps x `batch` sequences, 2 x LSTM 1024, projection + softmax on every row, perplexity update
@@ -238,7 +344,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "images", "ptb"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "images", "ptb", "memops"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
                          "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
                          "for counter passes over a single kernel")
@@ -249,6 +355,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--recurrent-net", default="lstm", choices=["lstm", "rnn"], help="network of --workload ptb")
+    ap.add_argument("--dump-launches", default="", help="write the tile shape and k-split every convolution layer ran with (JSON) to this file")
+    ap.add_argument("--pin-launches", default="", help="run every convolution layer with the tile shape and k-split listed in this file "
+                    "(as written by --dump-launches) instead of searching: repeats another run's launches exactly, e.g. under counter collection")
     ap.add_argument("--graph", type=int, default=0, help="1: forward passes are replays of a recorded HIP graph, 0 (default): eager "
                     "launches (the passes are GPU-bound on this machine: both take the same time)")
     args = ap.parse_args()
@@ -264,6 +373,8 @@ def main():
         return image_input(args)
     if args.workload == "ptb":
         return recurrent_driver(args)
+    if args.workload == "memops":
+        return memory_bound_kernels(args)
 
     from nebula_amd.net import Network
 
@@ -281,6 +392,12 @@ def main():
     n_in = net.batch_size * net.input_size
     x = (rng.random(n_in, dtype=np.float32) if xdist == "uniform" else rng.standard_normal(n_in).astype(np.float32))
     net.set_input(x)                     # resident in HBM before the timed region
+    conv_layers = [i for i in range(net.num_layers) if net.layer_info(i)["kind"] == "convolutional_layer"]
+    if args.pin_launches:
+        pinned = json.load(open(args.pin_launches))
+        assert [p["layer"] for p in pinned] == conv_layers, "--pin-launches: the file lists other layers than this workload has"
+        for p in pinned:
+            net.conv_pin_launch(p["layer"], p["variant"], p["k_slices"] if p["k_slices"] > 1 else 0)
     use_graph = args.graph == 1
     if use_graph:
         net.set_graph(True)              # pass 1 eager, pass 2 recorded, replays from pass 3 (all inside the warm-up)
@@ -298,6 +415,23 @@ def main():
     net.sync()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
+    # what was timed must be a forward pass: finite outputs, and probability rows that sum to one
+    final = net.output(net.num_layers - 1 if net.layer_info(net.num_layers - 1)["kind"] != "cost_layer" else net.num_layers - 2)
+    assert np.isfinite(final).all(), "bench.py: the timed network produced non-finite outputs"
+    if any(net.layer_info(i)["kind"] == "softmax_layer" for i in range(net.num_layers)):
+        sm = max(i for i in range(net.num_layers) if net.layer_info(i)["kind"] == "softmax_layer")
+        rows_out = batch if (args.workload == "lstm") else net.batch_size
+        probs = net.output(sm).reshape(net.batch_size, -1)[:rows_out]
+        assert np.abs(probs.sum(1) - 1.0).max() < 1e-3, "bench.py: softmax rows of the timed network do not sum to 1"
+    # tile shape and k slices each convolution launch of the timed passes used (searched on the first pass unless pinned)
+    variant_names = ["128x128", "64x256", "96x256", "64x128", "64x64", "128x64", "strip"]
+    launches = []
+    for i in conv_layers:
+        v, g = net.conv_last_launch(i)
+        launches.append({"layer": i, "variant": v, "tile": variant_names[v] if 0 <= v < len(variant_names) else str(v), "k_slices": g})
+    if args.dump_launches:
+        with open(args.dump_launches, "w") as f:
+            json.dump(launches, f)
     units = batch                         # images (or sequences) per step
     value = units / (wall / args.steps)
     log("timed %d steps: wall %.3f ms/step, events %.3f ms/step" % (args.steps, ms_per_step, ev_ms / args.steps))
@@ -365,7 +499,9 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded",
-                   "launch": "hip graph replay" if use_graph and net.graph_active else "eager"},
+                   "launch": "hip graph replay" if use_graph and net.graph_active else "eager",
+                   "conv_launches": "pinned from " + os.path.basename(args.pin_launches) if args.pin_launches else "searched on the first pass",
+                   "conv_tiles": " ".join("%d:%s%s" % (p["layer"], p["tile"], "/%d" % p["k_slices"] if p["k_slices"] > 1 else "") for p in launches)},
         "roofline": roofline,
     }
 

@@ -110,7 +110,10 @@ int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *plan);
 /* Algorithmic FLOP of one forward at batch B (2*B*F*OH*OW*C*k*k) and the output dims. */
 int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, double *flop_per_image);
 /* Pick the tile shape by hand (tests / tuning); variant < 0 restores the built-in choice.
- * nbl_conv2d_num_variants() says how many exist. */
+ * nbl_conv2d_num_variants() says how many exist.  Layers with at most 4 input channels and a filter larger than 1x1
+ * (the first layer of an image network) have one more kernel, which builds the patch matrix from a strip of the
+ * image staged in LDS: variant == nbl_conv2d_num_variants() names it (NBL_EINVAL for a plan that does not qualify;
+ * it fuses no shortcut: nbl_conv2d_shortcut_fwd falls back to a tile shape). */
 int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
 /* k-split of launches whose tile count leaves CUs idle in the last round: the tiles of that round are
  * cut into slices along C*k*k, one block each, and a second small kernel adds the slices in slice order

@@ -817,6 +817,7 @@ struct nbl_conv_plan {
     int tuned_slices;           // 0 = unsplit, 1 = the cost model's slice count, 2..8 = that many
     float *ws_dev; size_t ws_bytes;   // partial sums of split launches (grown on demand)
     int last_variant, last_split;     // what the most recent launch used
+    nbl_strip_plan strip;             // layers with very few input channels: the kernel of conv_strip.hip, variant index NUM_VARIANTS
 };
 
 namespace {
@@ -905,6 +906,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
     p->split_mode = -1; p->tuned_slices = 0; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
     p->tuned_batch = 0; p->tuned_variant = -1;
+    p->strip.eligible = false; p->strip.otab_dev = NULL;
     p->wp_dev = NULL; p->wp_rows_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
     p->tap_major = ksize > 1 && ksize * ksize <= 31 && C % CONV_BK == 0;
 
@@ -941,12 +943,21 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
         nbl_conv2d_plan_destroy(ctx, p);
         return rc;
     }
+    nbl_strip_plan &sp = p->strip;
+    sp.C = (int)C; sp.H = (int)H; sp.W = (int)W; sp.F = (int)F; sp.k = (int)ksize; sp.stride = (int)stride; sp.pad = (int)pad;
+    sp.OH = (int)p->OH; sp.OW = (int)p->OW; sp.K = (int)p->K; sp.Kp = (int)p->Kp; sp.Mp = (int)p->Mp; sp.act = act;
+    sp.wq_dev = p->wp_dev; sp.g_dev = p->g_dev; sp.b_dev = p->b_dev;
+    if(!p->tap_major && (rc = nbl_conv_strip_pack(ctx, &sp)) != NBL_OK) {      // (its table follows the reference row order)
+        nbl_conv2d_plan_destroy(ctx, p);
+        return rc;
+    }
     *out = p;
     return NBL_OK;
 }
 
 int nbl_conv2d_plan_destroy(nbl_ctx *ctx, nbl_conv_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
+    nbl_conv_strip_destroy(ctx, &p->strip);
     nbl_free(ctx, p->ttab_dev);
     nbl_free(ctx, p->wp_dev); nbl_free(ctx, p->wp_rows_dev); nbl_free(ctx, p->ktab_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev);
     nbl_free(ctx, p->ws_dev);
@@ -963,7 +974,8 @@ int nbl_conv2d_plan_info(const nbl_conv_plan *p, unsigned *OH, unsigned *OW, dou
 }
 
 int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
-    if(!p || variant >= NUM_VARIANTS) return NBL_EINVAL;
+    // index NUM_VARIANTS names the strip kernel of layers with very few input channels (only where the plan qualifies)
+    if(!p || variant > NUM_VARIANTS || (variant == NUM_VARIANTS && !p->strip.eligible)) return NBL_EINVAL;
     p->variant = variant < 0 ? -1 : variant;
     return NBL_OK;
 }
@@ -987,6 +999,12 @@ struct ConvResidual { const float *res; unsigned c, h, w; int post_act; };
 // slices: 0 = unsplit, 1 = k-split with the cost model's slice count, 2..8 = k-split with that many slices
 static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B, int v,
                        int slices, const ConvResidual *rs) {
+    if(v == NUM_VARIANTS) {           // strip kernel: whole tiles only, no fused shortcut
+        if(rs || !p->strip.eligible) return nbl_fail(ctx, NBL_EINVAL, "nbl_conv2d_fwd: internal: strip kernel asked for a layer it does not take");
+        const int rc = nbl_conv_strip_forward(ctx, &p->strip, x_dev, y_dev, B);
+        if(rc == NBL_OK) { p->last_variant = v; p->last_split = 1; }
+        return rc;
+    }
     const size_t in_elems = (size_t)B * p->C * p->H * p->W;
     const size_t npix = (size_t)B * p->OH * p->OW;
     const Variant &var = VARIANTS[v];
@@ -1092,6 +1110,7 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
             if(sp.split > 1 || p->split_mode > 0) cand.push_back({ v, slices, 0.0f });
         }
     }
+    if(p->strip.eligible && !rs) cand.push_back({ NUM_VARIANTS, 0, 0.0f });
     const int fallback = choose_variant(p, B * p->OH * p->OW, ctx->num_cu);
     if(cand.empty()) { p->tuned_batch = B; p->tuned_variant = fallback; p->tuned_slices = p->split_mode > 0 ? p->split_mode : 0; return NBL_OK; }
 
@@ -1151,6 +1170,7 @@ static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_
         v = p->tuned_variant;
         slices = p->tuned_slices;
     }
+    if(v == NUM_VARIANTS && rs) { v = choose_variant(p, (unsigned)npix, ctx->num_cu); slices = 0; }     // the strip kernel fuses no shortcut
     return conv_launch(ctx, p, x_dev, y_dev, B, v, slices, rs);
 }
 

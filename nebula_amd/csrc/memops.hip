@@ -236,9 +236,10 @@ __global__ void shortcut_general_kernel(const float *__restrict__ prev, const fl
 }
 
 // ---- softmax -------------------------------------------------------------------------------------
-// One block per row (softmax_layer.cc:85-106): row maximum, e = exp(x - max) evaluated in double and
-// rounded to float as the CPU code does, sum, divide.  The sum is a tree over floats where the CPU
-// code adds left to right; the difference is far inside the 1e-4 tolerance of this layer.
+// One block per row (softmax_layer.cc:85-106): row maximum, e = exp(x - max), sum, divide.  The CPU code evaluates
+// exp in double and rounds to float; here it is the single-precision expf (within an ulp or two of that, against a
+// layer tolerance of 1e-4): the double-precision exp held the 4096 x 10000 step of the recurrent driver to 45 % of
+// the memory rate.  The sum is a tree over floats where the CPU code adds left to right.
 __device__ __forceinline__ float wave_max(float v) {
     for(int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
@@ -246,6 +247,50 @@ __device__ __forceinline__ float wave_max(float v) {
 __device__ __forceinline__ float wave_sum(float v) {
     for(int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
+}
+__device__ __forceinline__ float softmax_exp(float d) { return expf(d); }
+
+// Rows whose length is a multiple of 4 and whose start is 16-byte aligned, up to 1024 * PER4 entries: a thread keeps
+// PER4 pieces of four adjacent entries in registers (pieces tid, tid + 256, ...), so the row moves as 16-byte loads
+// and stores, once each way.
+template<int PER4>
+__global__ __launch_bounds__(256) void softmax_row_vec4_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
+    typedef float vec4 __attribute__((ext_vector_type(4)));
+    __shared__ float red[4];
+    const vec4 *in = reinterpret_cast<const vec4*>(x + (size_t)blockIdx.x * n);
+    vec4 *out = reinterpret_cast<vec4*>(y + (size_t)blockIdx.x * n);
+    const unsigned n4 = n / 4;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    vec4 v[PER4];
+    float m = -FLT_MAX;
+    #pragma unroll
+    for(int i = 0; i < PER4; i++) {
+        const unsigned j = tid + i * 256;
+        v[i] = j < n4 ? in[j] : vec4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+        m = fmaxf(fmaxf(m, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+    }
+    m = wave_max(m);
+    if(lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float s = 0.0f;
+    #pragma unroll
+    for(int i = 0; i < PER4; i++) {
+        if(tid + i * 256 < n4) {
+            #pragma unroll
+            for(int c = 0; c < 4; c++) { v[i][c] = softmax_exp(v[i][c] - m); s += v[i][c]; }
+        }
+    }
+    s = wave_sum(s);
+    if(lane == 0) red[wave] = s;
+    __syncthreads();
+    s = (red[0] + red[1]) + (red[2] + red[3]);
+    #pragma unroll
+    for(int i = 0; i < PER4; i++) {
+        const unsigned j = tid + i * 256;
+        if(j < n4) out[j] = vec4{v[i][0] / s, v[i][1] / s, v[i][2] / s, v[i][3] / s};
+    }
 }
 
 // Rows of up to THREADS * PER entries: a thread keeps its PER entries (columns tid, tid + THREADS, ...) in
@@ -278,7 +323,7 @@ __global__ __launch_bounds__(THREADS) void softmax_row_in_registers_kernel(const
     for(int i = 0; i < PER; i++) {
         const unsigned j = tid + i * THREADS;
         if(j < n) {
-            v[i] = (float)exp((double)(v[i] - m));
+            v[i] = softmax_exp(v[i] - m);
             s += v[i];
         }
     }
@@ -300,8 +345,7 @@ __global__ __launch_bounds__(THREADS) void softmax_row_in_registers_kernel(const
     }
 }
 
-// One block of THREADS threads per row of any length (long rows take 1024 threads: the exp is double precision and
-// there are only as many blocks as rows); the row is read three times and written twice.
+// One block of THREADS threads per row of any length; the row is read three times and written twice.
 template<int THREADS>
 __global__ __launch_bounds__(THREADS) void softmax_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
     constexpr int WAVES = THREADS / 64;
@@ -320,7 +364,7 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(const float *__restric
     __syncthreads();
     float s = 0.0f;
     for(unsigned j = tid; j < n; j += THREADS) {
-        const float e = (float)exp((double)(in[j] - m));
+        const float e = softmax_exp(in[j] - m);
         out[j] = e;
         s += e;
     }
@@ -352,26 +396,40 @@ __global__ void activation_kernel(float *__restrict__ x, size_t n, int act) {
     }
 }
 
-// y[b][c][s] = y * g[c] + b[c]   (bias only: g == NULL)
+// y[b][c][s] = y * g[c] + b[c]   (bias only: g == NULL).  VEC = 4 needs size % 4 == 0 and a 16-byte aligned tensor:
+// the four elements of a piece then share their channel.
+template<int VEC>
 __global__ void channel_affine_kernel(float *__restrict__ y, const float *__restrict__ g, const float *__restrict__ b,
                                       size_t total, unsigned channel, unsigned size) {
-    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    typedef float __attribute__((ext_vector_type(VEC))) vec;
+    const size_t e = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if(e >= total) return;
     const unsigned c = (unsigned)((e / size) % channel);
-    y[e] = g ? y[e] * g[c] + b[c] : y[e] + b[c];
+    const float bc = b[c], gc = g ? g[c] : 1.0f;
+    vec v = *reinterpret_cast<vec*>(y + e);
+    #pragma unroll
+    for(int i = 0; i < VEC; i++) v[i] = g ? v[i] * gc + bc : v[i] + bc;
+    *reinterpret_cast<vec*>(y + e) = v;
 }
 
 // y = (float)((double)(y - mean[c]) / (sqrt(var[c]) + 1e-5)) * scale[c], the two CPU passes of
-// common/batchnorm.cc:58-97 in one.
+// common/batchnorm.cc:58-97 in one.  The quotient is formed as a product with the channel's reciprocal in double,
+// one double rounding away from the CPU's division before the rounding to float (the same float in all but about
+// one case in 2^29).
+template<int VEC>
 __global__ void batchnorm_inference_kernel(float *__restrict__ y, const float *__restrict__ mean,
                                            const float *__restrict__ var, const float *__restrict__ scale,
                                            size_t total, unsigned channel, unsigned size) {
-    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    typedef float __attribute__((ext_vector_type(VEC))) vec;
+    const size_t e = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if(e >= total) return;
     const unsigned c = (unsigned)((e / size) % channel);
-    const float centered = __fsub_rn(y[e], mean[c]);
-    const float normed = (float)((double)centered / (sqrt((double)var[c]) + 0.00001));
-    y[e] = __fmul_rn(normed, scale[c]);
+    const float mc = mean[c], sc = scale[c];
+    const double r = 1.0 / (sqrt((double)var[c]) + 0.00001);
+    vec v = *reinterpret_cast<vec*>(y + e);
+    #pragma unroll
+    for(int i = 0; i < VEC; i++) v[i] = __fmul_rn((float)((double)__fsub_rn(v[i], mc) * r), sc);
+    *reinterpret_cast<vec*>(y + e) = v;
 }
 
 
@@ -593,7 +651,15 @@ int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned row
     if(!ctx) return NBL_EINVAL;
     NBL_REQUIRE(ctx, x_dev && y_dev, "nbl_softmax_fwd: NULL pointer");
     if(rows == 0 || n == 0) return NBL_OK;
-    if(n <= 1024)       hipLaunchKernelGGL((softmax_row_in_registers_kernel<256, 4>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
+    if(n % 4 == 0 && n <= 16384 && (((size_t)x_dev | (size_t)y_dev) & 15) == 0) {
+        const unsigned per4 = nbl_div_up(n / 4, 256);
+#define NBL_SOFTMAX_VEC(P) hipLaunchKernelGGL((softmax_row_vec4_kernel<P>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n)
+        if(per4 <= 1) NBL_SOFTMAX_VEC(1); else if(per4 <= 2) NBL_SOFTMAX_VEC(2); else if(per4 <= 4) NBL_SOFTMAX_VEC(4);
+        else if(per4 <= 6) NBL_SOFTMAX_VEC(6); else if(per4 <= 8) NBL_SOFTMAX_VEC(8); else if(per4 <= 10) NBL_SOFTMAX_VEC(10);
+        else if(per4 <= 12) NBL_SOFTMAX_VEC(12); else NBL_SOFTMAX_VEC(16);
+#undef NBL_SOFTMAX_VEC
+    }
+    else if(n <= 1024)  hipLaunchKernelGGL((softmax_row_in_registers_kernel<256, 4>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
     else if(n <= 2048)  hipLaunchKernelGGL((softmax_row_in_registers_kernel<256, 8>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n);
     else if(n <= 16384) hipLaunchKernelGGL((softmax_row_in_registers_kernel<1024, 16>), dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
     else                hipLaunchKernelGGL(softmax_kernel<1024>, dim3(rows), dim3(1024), 0, ctx->stream, x_dev, y_dev, n);
@@ -620,8 +686,12 @@ int nbl_forward_bias(nbl_ctx *ctx, float *y_dev, const float *bias_dev,
     NBL_REQUIRE(ctx, y_dev && bias_dev, "nbl_forward_bias: NULL pointer");
     const size_t total = (size_t)batch * channel * size;
     if(total == 0) return NBL_OK;
-    hipLaunchKernelGGL(channel_affine_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
-                       y_dev, (const float*)NULL, bias_dev, total, channel, size);
+    if(size % 4 == 0 && ((size_t)y_dev & 15) == 0)
+        hipLaunchKernelGGL(channel_affine_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
+                           y_dev, (const float*)NULL, bias_dev, total, channel, size);
+    else
+        hipLaunchKernelGGL(channel_affine_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                           y_dev, (const float*)NULL, bias_dev, total, channel, size);
     NBL_LAUNCH_CHECK(ctx, "channel_affine_kernel");
     return NBL_OK;
 }
@@ -632,8 +702,12 @@ int nbl_batchnorm_inference(nbl_ctx *ctx, float *y_dev, const float *mean_dev, c
     NBL_REQUIRE(ctx, y_dev && mean_dev && var_dev && scale_dev, "nbl_batchnorm_inference: NULL pointer");
     const size_t total = (size_t)batch * channel * size;
     if(total == 0) return NBL_OK;
-    hipLaunchKernelGGL(batchnorm_inference_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
-                       y_dev, mean_dev, var_dev, scale_dev, total, channel, size);
+    if(size % 4 == 0 && ((size_t)y_dev & 15) == 0)
+        hipLaunchKernelGGL(batchnorm_inference_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
+                           y_dev, mean_dev, var_dev, scale_dev, total, channel, size);
+    else
+        hipLaunchKernelGGL(batchnorm_inference_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                           y_dev, mean_dev, var_dev, scale_dev, total, channel, size);
     NBL_LAUNCH_CHECK(ctx, "batchnorm_inference_kernel");
     return NBL_OK;
 }

@@ -89,3 +89,20 @@ static inline bool nbl_act_valid(int act) { return act > NBL_ACT_UNDEFINED && ac
 // Without batchnorm g is 1 and b is the bias.
 void nbl_fold_batchnorm(const float *bias, const float *scale, const float *mean, const float *var,
                         unsigned n, float *g_out, float *b_out);
+
+// Convolutions with very few input channels (the first layer of an image network: 3 channels, a large filter):
+// their patch rows come from a handful of input rows, so a block stages that strip of the image in LDS once and
+// feeds the matrix cores from it (csrc/conv_strip.hip).  Filled by nbl_conv2d_pack when the layer qualifies.
+struct nbl_strip_plan {
+    bool eligible;
+    int C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp, act;
+    int mt;                 // 32-filter MFMA tiles per wave (block tile = 32*mt filters x 128 pixels)
+    int rows, pitch;        // strip: input rows a block may need, floats per row (W + 2*pad)
+    int *otab_dev;          // [Kp] strip offset of every patch row; padding rows point at a zero word behind the strip
+    const float *wq_dev, *g_dev, *b_dev;     // packed weights [Kp / 4][Mp][4], per-filter multiply-add
+    size_t lds_bytes;
+};
+// Builds the offset table (host side of the plan); returns NBL_OK and leaves eligible = false when the layer does not qualify.
+int nbl_conv_strip_pack(nbl_ctx *ctx, nbl_strip_plan *sp);
+int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *x_dev, float *y_dev, unsigned B);
+void nbl_conv_strip_destroy(nbl_ctx *ctx, nbl_strip_plan *sp);

@@ -60,6 +60,12 @@ CONV = [
     (1, 5, 9, 11, 130, 5, 1, 2, False, "logistic"),       # F > one m-tile, ragged K
     (4, 32, 7, 7, 96, 3, 1, 1, True, "linear"),
     (2, 4, 6, 6, 3, 2, 2, 1, False, "tanh"),
+    # very few channels: the strip kernel's cases -- several tiles per image with a ragged last one, 2 and 3 filter
+    # tiles per wave, two filter tiles per block, one channel
+    (3, 3, 61, 45, 70, 7, 2, 3, True, "leaky"),
+    (2, 3, 75, 75, 96, 11, 4, 0, False, "relu"),
+    (2, 1, 33, 20, 150, 5, 1, 2, True, "logistic"),
+    (5, 2, 16, 23, 9, 3, 1, 1, False, "linear"),
 ]
 
 
@@ -79,7 +85,12 @@ def test_conv_matches_oracle(ctx, case):
     want = ob.conv_forward(x, w, bias, bnp, s, p, act)
     plan = ctx.conv_pack(w, bias, bnp, H=H, W=W, stride=s, pad=p, act=act)
     dx = ctx.array(x)
-    for v in [-1] + list(range(hip.lib().nbl_conv2d_num_variants())):
+    nv = hip.lib().nbl_conv2d_num_variants()
+    variants = [-1] + list(range(nv))
+    if hip.lib().nbl_conv2d_plan_set_variant(plan.p, nv) == 0:      # layers with very few channels also have the strip kernel
+        variants.append(nv)
+    assert (nv in variants) == (Cc <= 4 and k > 1), "strip kernel eligibility changed for %r" % (case,)
+    for v in variants:
         announce("conv variant", v)
         plan.set_variant(v)
         got = plan(dx).numpy()
