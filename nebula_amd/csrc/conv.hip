@@ -57,6 +57,7 @@ struct ConvArgs {
     // to ws[p][f][n - n_start]; conv_split_finish_kernel adds the parts and applies the epilogue
     int whole_tiles, split, n_start, n_tail;
     int units;     // whole_tiles + (tiles - whole_tiles) * split: work units of the launch
+    int xcd_group; // consecutive pixel tiles that share an XCD (see the block index mapping in the kernel)
     float *ws;
     // tap-major layers: one entry per k-tile, {byte offset of the tile's tap in channel c0's plane +
     // c0*H*W*4, 31 - tap index (the left shift that brings the tap's bit of a pixel's outside mask to
@@ -189,13 +190,17 @@ void conv_igemm_kernel(const ConvArgs a) {
     const int nkt = a.Kp / BK;        // even: Kp is a multiple of 2*BK
     // Workgroups are dealt to the 8 XCDs round robin by index, and each XCD has its own L2.  The work
     // units are therefore renumbered so that a run of tiles_m consecutive units (the filter tiles of one
-    // pixel tile, which read the same input) lands on one XCD, runs being dealt round robin in turn.
+    // pixel tile, which read the same input) lands on one XCD, and so do xcd_group consecutive runs: neighbouring
+    // pixel tiles of a 3x3 layer read each other's rows (every input row of a 56-wide plane is needed by three
+    // 64-pixel tiles), and with neighbours on different XCDs each of them fetched those rows from memory again.
+    // Groups of runs are dealt round robin in turn.
     int tile;
     {
-        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run = slot / (unsigned)a.tiles_m,
-                       within = slot - run * (unsigned)a.tiles_m;
-        const unsigned unit = (run * 8u + xcd) * (unsigned)a.tiles_m + within;
-        if(unit >= (unsigned)a.units) return;         // the grid is padded to whole rounds of runs
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = slot / (unsigned)a.tiles_m,
+                       within = slot - run_local * (unsigned)a.tiles_m;
+        const unsigned G = (unsigned)a.xcd_group, group_local = run_local / G, j = run_local - group_local * G;
+        const unsigned unit = (((group_local * 8u + xcd) * G) + j) * (unsigned)a.tiles_m + within;
+        if(unit >= (unsigned)a.units) return;         // the grid is padded to whole rounds of groups
         tile = (int)unit;
     }
     const int unit = tile;
@@ -1068,7 +1073,11 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
         }
     }
     a.units = (int)grid;
-    const size_t round = 8u * (size_t)a.tiles_m;
+    {
+        const size_t runs = nbl_div_up_sz(grid, (size_t)a.tiles_m);
+        a.xcd_group = (int)std::max<size_t>(1, std::min<size_t>(8, runs / 16));      // every XCD still gets at least two groups
+    }
+    const size_t round = 8u * (size_t)a.xcd_group * (size_t)a.tiles_m;
     grid = nbl_div_up_sz(grid, round) * round;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)grid), dim3(var.threads), 0,

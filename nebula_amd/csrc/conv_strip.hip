@@ -37,6 +37,7 @@ struct StripArgs {
     int Kp, Mp, tiles_m, tiles_per_image;
     int rows, pitch;
     int act;
+    int runs;               // pixel tiles of the launch (tiles_per_image * batch)
 };
 
 // (MT = 2: five blocks per CU fit its LDS use when the registers allow it too -- 6272 tiles of the 7x7 stem at batch 64
@@ -51,7 +52,16 @@ void conv_strip_kernel(const StripArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // uniform, and known to be: per-row buffer descriptors are built from it
-    const int tm = blockIdx.x % a.tiles_m, tn = blockIdx.x / a.tiles_m;
+    // Workgroups go to the 8 XCDs round robin by index and each XCD has its own L2: eight consecutive pixel tiles
+    // (whose strips overlap in all but a row or two) share an XCD, groups of eight are dealt round robin.
+    int tm, tn;
+    {
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = slot / (unsigned)a.tiles_m,
+                       within = slot - run_local * (unsigned)a.tiles_m;
+        const unsigned run = ((run_local >> 3) * 8u + xcd) * 8u + (run_local & 7u);
+        if(run >= (unsigned)a.runs) return;             // the grid is padded to whole rounds of groups
+        tm = (int)within; tn = (int)run;
+    }
     const int img = tn / a.tiles_per_image, p0 = (tn - img * a.tiles_per_image) * STRIP_BN;
     const int m0 = tm * MT * 32;
     const int oh0 = p0 / a.OW, ih0 = oh0 * a.stride - a.pad;
@@ -253,7 +263,8 @@ int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *
     a.Kp = sp->Kp; a.Mp = sp->Mp; a.tiles_m = (int)nbl_div_up(sp->F, sp->mt * 32);
     a.tiles_per_image = (int)nbl_div_up(a.OHW, STRIP_BN);
     a.rows = sp->rows; a.pitch = sp->pitch; a.act = sp->act;
-    const size_t grid = (size_t)a.tiles_m * a.tiles_per_image * B;
+    a.runs = a.tiles_per_image * (int)B;
+    const size_t grid = nbl_div_up_sz((size_t)a.runs, 64) * 64 * a.tiles_m;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     const bool fast = sp->act == NBL_ACT_RELU || sp->act == NBL_ACT_LINEAR || sp->act == NBL_ACT_LEAKY || sp->act == NBL_ACT_RELIE;
     // more than 64 KB of dynamic LDS has to be asked for, once per kernel
