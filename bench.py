@@ -143,12 +143,17 @@ def single_conv(args):
     plan.set_split(args.conv_split)
     x = ctx.array(rng.standard_normal((B, C_, H, W)).astype(np.float32))
     y = ctx.empty((B, F, plan.OH, plan.OW))
+    if args.conv_residual:              # the layer as ResNet runs it: the following shortcut fused into the epilogue
+        conn = ctx.array(rng.standard_normal((B, F, plan.OH, plan.OW)).astype(np.float32))
+        run = lambda: plan.with_shortcut(x, conn, "relu", out=y)
+    else:
+        run = lambda: plan(x, out=y)
     for _ in range(args.warmup):
-        plan(x, out=y)
+        run()
     ctx.sync()
     ctx.timer_start()
     for _ in range(args.steps):
-        plan(x, out=y)
+        run()
     ms = ctx.timer_stop() / args.steps
     variant, parts = plan.last_launch()
     flop = plan.flop_per_image * B
@@ -351,6 +356,7 @@ def main():
     ap.add_argument("--conv-shape", default="512,28,28,256,1,1,0", help="C,H,W,F,k,stride,pad of --workload conv")
     ap.add_argument("--conv-variant", type=int, default=-1, help="tile shape index of --workload conv (-1: searched)")
     ap.add_argument("--conv-split", type=int, default=-1, help="k-split mode of --workload conv (-1 searched, 0 off, 1 model)")
+    ap.add_argument("--conv-residual", type=int, default=0, help="1: --workload conv adds a same-shape residual and relu in the epilogue (fused shortcut)")
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")

@@ -39,6 +39,31 @@ constexpr int CONV_BK = 16;          // k-tile depth (8 MFMA k-steps)
 constexpr int CONV_MP_ALIGN = 384;   // lcm of the BM values below
 constexpr int KTAB_PAD_TAP = 0x4000; // tap row of a padded table entry: always outside the image
 
+// Division by a number known on the host: q = umulhi(n, mul) >> shr for n < 2^31 (mul = ceil(2^(31 + ceil(log2 d)) / d)).
+// A runtime integer division costs some 25 ordinary vector instructions, and the block's set-up has half a dozen of
+// them; ordinary vector instructions are paid for in matrix-pipe time, which matters for layers with few patch rows.
+struct FastDiv {
+    unsigned mul, shr, d;
+    __host__ __device__ __forceinline__ unsigned div(unsigned n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return d == 1u ? n : __umulhi(n, mul) >> shr;
+#else
+        return n / d;
+#endif
+    }
+};
+inline FastDiv make_fastdiv(unsigned d) {
+    FastDiv f; f.d = d; f.mul = 0; f.shr = 0;
+    if(d > 1) {
+        unsigned lg = 0;
+        while((1ull << lg) < d) lg++;
+        const unsigned p = 31 + lg;
+        f.mul = (unsigned)(((1ull << p) + d - 1) / d);
+        f.shr = p - 32;
+    }
+    return f;
+}
+
 struct ConvArgs {
     const float *x; const float *wp; const int2 *ktab; const float *g; const float *b; float *y;
     int H, W, F, OW, OHW, CHW, stride, pad;
@@ -57,7 +82,8 @@ struct ConvArgs {
     // to ws[p][f][n - n_start]; conv_split_finish_kernel adds the parts and applies the epilogue
     int whole_tiles, split, n_start, n_tail;
     int units;     // whole_tiles + (tiles - whole_tiles) * split: work units of the launch
-    int xcd_group; // consecutive pixel tiles that share an XCD (see the block index mapping in the kernel)
+    int xcd_group_log2; // log2 of the consecutive pixel tiles that share an XCD (see the block index mapping in the kernel)
+    FastDiv div_tiles_m, div_ohw, div_ow, div_split;
     float *ws;
     // tap-major layers: one entry per k-tile, {byte offset of the tile's tap in channel c0's plane +
     // c0*H*W*4, 31 - tap index (the left shift that brings the tap's bit of a pixel's outside mask to
@@ -86,11 +112,11 @@ struct PixelCoord { int xbase; int ih0; int iw0; };
 // Pixel column n -> input base offset and top-left tap coordinate.  n >= N gives a coordinate
 // that fails every bounds test.
 __device__ __forceinline__ PixelCoord conv_pixel(int n, int N, int OHW, int OW, int stride, int pad,
-                                                 int CHW, int W) {
+                                                 int CHW, int W, const FastDiv &dohw, const FastDiv &dow) {
     PixelCoord p;
     if(n < N) {
-        const int b = n / OHW, pix = n - b * OHW;
-        const int oh = pix / OW, ow = pix - oh * OW;
+        const int b = (int)dohw.div((unsigned)n), pix = n - b * OHW;
+        const int oh = (int)dow.div((unsigned)pix), ow = pix - oh * OW;
         p.ih0 = oh * stride - pad;
         p.iw0 = ow * stride - pad;
         p.xbase = b * CHW + p.ih0 * W + p.iw0;
@@ -196,10 +222,10 @@ void conv_igemm_kernel(const ConvArgs a) {
     // Groups of runs are dealt round robin in turn.
     int tile;
     {
-        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = slot / (unsigned)a.tiles_m,
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = a.div_tiles_m.div(slot),
                        within = slot - run_local * (unsigned)a.tiles_m;
-        const unsigned G = (unsigned)a.xcd_group, group_local = run_local / G, j = run_local - group_local * G;
-        const unsigned unit = (((group_local * 8u + xcd) * G) + j) * (unsigned)a.tiles_m + within;
+        const unsigned gl = (unsigned)a.xcd_group_log2, group_local = run_local >> gl, j = run_local & ((1u << gl) - 1u);
+        const unsigned unit = ((((group_local << 3) + xcd) << gl) + j) * (unsigned)a.tiles_m + within;
         if(unit >= (unsigned)a.units) return;         // the grid is padded to whole rounds of groups
         tile = (int)unit;
     }
@@ -207,10 +233,11 @@ void conv_igemm_kernel(const ConvArgs a) {
     int part = 0, kt_begin = 0, kt_end = nkt;
     if(tile >= a.whole_tiles) {
         const int u = tile - a.whole_tiles, pairs = nkt / 2;
-        tile = a.whole_tiles + u / a.split;
-        part = u % a.split;
-        kt_begin = 2 * (part * pairs / a.split);
-        kt_end = 2 * ((part + 1) * pairs / a.split);
+        const int ut = (int)a.div_split.div((unsigned)u);
+        tile = a.whole_tiles + ut;
+        part = u - ut * a.split;
+        kt_begin = 2 * (int)a.div_split.div((unsigned)(part * pairs));
+        kt_end = 2 * (int)a.div_split.div((unsigned)((part + 1) * pairs));
     }
     const bool split_block = unit >= a.whole_tiles;
 
@@ -224,16 +251,17 @@ void conv_igemm_kernel(const ConvArgs a) {
 
     // ---- load side state: the k-tile the next global loads belong to ----
     int ld_kt = kt_begin;
-    const int ld_m0 = (tile % a.tiles_m) * BM;
+    const int tile_n = (int)a.div_tiles_m.div((unsigned)tile), tile_m = tile - tile_n * a.tiles_m;
+    const int ld_m0 = tile_m * BM;
     PixelCoord px;
     unsigned xoff;
     {
-        const int n0 = (tile / a.tiles_m) * BN;
+        const int n0 = tile_n * BN;
         // VEC4 reads with plain 16-byte global loads, so its addresses must be real: a column group past
         // the last pixel re-reads the last group (its results are never stored), a row past the last patch
         // row re-reads the last row and is zeroed when the tile is written to LDS.
         const int ncol_first = VEC4 ? min(n0 + ncol * 4, a.N - 4) : n0 + ncol;
-        px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W);
+        px = conv_pixel(ncol_first, a.N, a.OHW, a.OW, a.stride, a.pad, a.CHW, a.W, a.div_ohw, a.div_ow);
         // byte offset of the pixel's top-left tap; a column past the last pixel is out of range for every k
         xoff = px.ih0 > -(1 << 29) ? (unsigned)px.xbase * 4u : OOB_OFFSET;
     }
@@ -416,14 +444,19 @@ void conv_igemm_kernel(const ConvArgs a) {
     // (forced inline: called from four places, and as a real call it would take the accumulators through memory)
     auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff, unsigned roff, int act, int post_act)
                           __attribute__((always_inline)) {
+        // sloped: 0 relu / linear through selects on uniform flags, 1 leaky / relie as well, 2 the ReLU network's two
+        //         cases resolved at compile time: relu without a residual, or linear + residual + relu (one max each)
         // with_residual: 0 none, 1 at the output's own offsets (same shape), 2 at offsets of its own
-        constexpr bool SLOPED = decltype(sloped)::value, RES = decltype(with_residual)::value != 0,
-                       RES_OWN = decltype(with_residual)::value == 2;
+        constexpr bool SLOPED = decltype(sloped)::value == 1, RELU_NET = decltype(sloped)::value == 2,
+                       RES = decltype(with_residual)::value != 0, RES_OWN = decltype(with_residual)::value == 2;
         typedef float __attribute__((ext_vector_type(NT))) pixvec;
         const unsigned row_bytes = (unsigned)a.OHW * 4u;
-        char *__restrict__ yb = reinterpret_cast<char*>(a.y);
-        const char *__restrict__ rb = reinterpret_cast<const char*>(a.res);
         const unsigned res_row_bytes = (unsigned)a.res_hw * 4u;
+        // Output rows (and residual rows) go through buffer descriptors: the lane's own offset is a constant vector
+        // offset, the row's offset is uniform and rides in the scalar offset -- no address arithmetic per row.  (Both
+        // tensors are below 4 GiB here, which is what selects this epilogue.)
+        const __amdgpu_buffer_rsrc_t yres = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, (int)0xffffffffu, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(RES ? a.res : a.y), 0, (int)0xffffffffu, 0x00020000);
         // per-filter constants one group of rows ahead of their use
         vec4f gv[2][MT], bv[2][MT];
         auto load_constants = [&](int q) {
@@ -440,9 +473,11 @@ void conv_igemm_kernel(const ConvArgs a) {
             pixvec rv[4 * MT];
             if(RES) {
                 #pragma unroll
-                for(int e = 0; e < 4 * MT; e++)
-                    rv[e] = *reinterpret_cast<const pixvec*>(rb + (RES_OWN ? (size_t)(roff + (unsigned)(q * 8 * MT + e) * res_row_bytes)
-                                                                           : (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes)));
+                for(int e = 0; e < 4 * MT; e++) {
+                    const unsigned row = (unsigned)(q * 8 * MT + e) * (RES_OWN ? res_row_bytes : row_bytes);       // uniform
+                    if constexpr(NT == 1) rv[e][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rres, (int)(RES_OWN ? roff : yoff), (int)row, 0));
+                    else rv[e] = __builtin_bit_cast(pixvec, __builtin_amdgcn_raw_buffer_load_b64(rres, (int)(RES_OWN ? roff : yoff), (int)row, 0));
+                }
             }
             #pragma unroll
             for(int e = 0; e < 4 * MT; e++) {
@@ -451,10 +486,19 @@ void conv_igemm_kernel(const ConvArgs a) {
                 pixvec o;
                 #pragma unroll
                 for(int j = 0; j < NT; j++) {
-                    o[j] = conv_cheap_activation<SLOPED>(__builtin_fmaf(acc[i][j][q * 4 + rr], ge, be), act);
-                    if(RES) o[j] = conv_cheap_activation<SLOPED>(__fadd_rn(o[j], rv[e][j]), post_act);
+                    const float t = __builtin_fmaf(acc[i][j][q * 4 + rr], ge, be);
+                    if(RELU_NET) {
+                        const float u = RES ? __fadd_rn(t, rv[e][j]) : t;
+                        o[j] = u > 0.0f ? u : 0.0f;
+                    } else {
+                        o[j] = conv_cheap_activation<SLOPED>(t, act);
+                        if(RES) o[j] = conv_cheap_activation<SLOPED>(__fadd_rn(o[j], rv[e][j]), post_act);
+                    }
                 }
-                *reinterpret_cast<pixvec*>(yb + (size_t)(yoff + (unsigned)(q * 8 * MT + e) * row_bytes)) = o;
+                const unsigned row = (unsigned)(q * 8 * MT + e) * row_bytes;       // uniform
+                typedef int __attribute__((ext_vector_type(2))) int2v;
+                if constexpr(NT == 1) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, o[0]), yres, (int)yoff, (int)row, 0);
+                else __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(int2v, o), yres, (int)yoff, (int)row, 0);
             }
         }
     };
@@ -464,11 +508,10 @@ void conv_igemm_kernel(const ConvArgs a) {
     // column lane%32; with the interleaving above that is filter row*MT + i and pixel (lane%32)*NT + j
     // of the wave's sub-tile.
     auto epilogue = [&](int tile) {
-        const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
-        const int m0 = tm * BM, n0 = tn * BN;
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
         const int nbase = n0 + wn * NT * 32 + l32 * NT;
         if(nbase >= a.N) return;
-        const int b0 = nbase / a.OHW, pix0 = nbase - b0 * a.OHW;
+        const int b0 = (int)a.div_ohw.div((unsigned)nbase), pix0 = nbase - b0 * a.OHW;
         // Short epilogue: every filter row of the tile exists, the lane's NT pixels are one aligned
         // vector (OH*OW even keeps pairs inside one image), and rows are reached as base pointer +
         // 32-bit offset, so a row costs one integer add besides its arithmetic.  An instruction spent
@@ -489,7 +532,7 @@ void conv_igemm_kernel(const ConvArgs a) {
             if(tile_res) {
                 unsigned rpix = (unsigned)pix0;
                 if(a.res_hw != a.OHW || a.res_stride != 1) {
-                    const int h = pix0 / a.OW, w = pix0 - h * a.OW;
+                    const int h = (int)a.div_ow.div((unsigned)pix0), w = pix0 - h * a.OW;
                     rpix = (unsigned)(h * a.res_stride * a.res_w + w * a.res_stride);
                 }
                 roff = ((unsigned)(b0 * a.res_c + f_lane) * (unsigned)a.res_hw + rpix) * 4u;
@@ -501,14 +544,22 @@ void conv_igemm_kernel(const ConvArgs a) {
             typedef std::integral_constant<int, 1> res_at_output;
             typedef std::integral_constant<int, 2> res_own;
             const bool res_same_shape = a.res_c == a.F && a.res_hw == a.OHW && a.res_stride == 1;   // uniform
-            if(a.short_epilogue == 1) {
-                if(!tile_res) short_epilogue(std::false_type(), no_res(), f_lane, yoff, roff, act, post_act);
-                else if(res_same_shape) short_epilogue(std::false_type(), res_at_output(), f_lane, yoff, roff, act, post_act);
-                else short_epilogue(std::false_type(), res_own(), f_lane, yoff, roff, act, post_act);
+            typedef std::integral_constant<int, 0> flags; typedef std::integral_constant<int, 1> slopes; typedef std::integral_constant<int, 2> relu_net;
+            // (uniform) the two forms a ReLU network's layers take: relu alone, or linear + residual + relu
+            const bool is_relu_net = a.short_epilogue == 1 && (tile_res ? act == NBL_ACT_LINEAR && post_act == NBL_ACT_RELU
+                                                                        : act == NBL_ACT_RELU && post_act == NBL_ACT_LINEAR);
+            if(is_relu_net) {
+                if(!tile_res) short_epilogue(relu_net(), no_res(), f_lane, yoff, roff, act, post_act);
+                else if(res_same_shape) short_epilogue(relu_net(), res_at_output(), f_lane, yoff, roff, act, post_act);
+                else short_epilogue(relu_net(), res_own(), f_lane, yoff, roff, act, post_act);
+            } else if(a.short_epilogue == 1) {
+                if(!tile_res) short_epilogue(flags(), no_res(), f_lane, yoff, roff, act, post_act);
+                else if(res_same_shape) short_epilogue(flags(), res_at_output(), f_lane, yoff, roff, act, post_act);
+                else short_epilogue(flags(), res_own(), f_lane, yoff, roff, act, post_act);
             } else {
-                if(!tile_res) short_epilogue(std::true_type(), no_res(), f_lane, yoff, roff, act, post_act);
-                else if(res_same_shape) short_epilogue(std::true_type(), res_at_output(), f_lane, yoff, roff, act, post_act);
-                else short_epilogue(std::true_type(), res_own(), f_lane, yoff, roff, act, post_act);
+                if(!tile_res) short_epilogue(slopes(), no_res(), f_lane, yoff, roff, act, post_act);
+                else if(res_same_shape) short_epilogue(slopes(), res_at_output(), f_lane, yoff, roff, act, post_act);
+                else short_epilogue(slopes(), res_own(), f_lane, yoff, roff, act, post_act);
             }
             return;
         }
@@ -634,7 +685,7 @@ void conv_igemm_kernel(const ConvArgs a) {
 
     // Raw sums of a split block: ws[part][f][n - n_start], the lane's NT pixels as one vector where aligned.
     auto store_partial = [&]() {
-        const int m0 = (tile % a.tiles_m) * BM, n0 = (tile / a.tiles_m) * BN;
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
         const int nbase = n0 + wn * NT * 32 + l32 * NT;
         if(nbase >= a.N) return;
         float *__restrict__ wsp = a.ws + (size_t)part * a.F * a.n_tail + (nbase - a.n_start);
@@ -734,11 +785,11 @@ __global__ void conv_split_finish_kernel(const ConvArgs a) {
 }
 
 __global__ void im2col_kernel(const float *__restrict__ x, const int2 *__restrict__ ktab, float *__restrict__ col,
-                              int K, int H, int W, int OW, int OHW, int stride, int pad) {
+                              int K, int H, int W, int OW, int OHW, int stride, int pad, FastDiv dohw, FastDiv dow) {
     const int pix = blockIdx.x * blockDim.x + threadIdx.x;
     const int kk = blockIdx.y;
     if(pix >= OHW || kk >= K) return;
-    const PixelCoord p = conv_pixel(pix, OHW, OHW, OW, stride, pad, 0, W);
+    const PixelCoord p = conv_pixel(pix, OHW, OHW, OW, stride, pad, 0, W, dohw, dow);
     col[(size_t)kk * OHW + pix] = conv_gather(x, p, ktab[kk], H, W);
 }
 
@@ -1075,9 +1126,10 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
     a.units = (int)grid;
     {
         const size_t runs = nbl_div_up_sz(grid, (size_t)a.tiles_m);
-        a.xcd_group = (int)std::max<size_t>(1, std::min<size_t>(8, runs / 16));      // every XCD still gets at least two groups
+        a.xcd_group_log2 = runs >= 128 ? 3 : runs >= 64 ? 2 : runs >= 32 ? 1 : 0;       // every XCD still gets at least two groups
     }
-    const size_t round = 8u * (size_t)a.xcd_group * (size_t)a.tiles_m;
+    a.div_split = make_fastdiv((unsigned)a.split); a.div_tiles_m = make_fastdiv((unsigned)a.tiles_m); a.div_ohw = make_fastdiv((unsigned)a.OHW); a.div_ow = make_fastdiv((unsigned)a.OW);
+    const size_t round = (8u << a.xcd_group_log2) * (size_t)a.tiles_m;
     grid = nbl_div_up_sz(grid, round) * round;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     hipLaunchKernelGGL(var.kernel[gather][fast_act ? 0 : 1], dim3((unsigned)grid), dim3(var.threads), 0,
@@ -1223,7 +1275,8 @@ int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigne
     if(rc != NBL_OK) return rc;
     if((rc = nbl_h2d(ctx, tab_dev, tab.data(), tab.size() * sizeof(int2))) != NBL_OK) { nbl_free(ctx, tab_dev); return rc; }
     hipLaunchKernelGGL(im2col_kernel, dim3(nbl_div_up(OH * OW, 256), K), dim3(256), 0, ctx->stream,
-                       x_dev, tab_dev, col_dev, (int)K, (int)H, (int)W, (int)OW, (int)(OH * OW), (int)stride, (int)pad);
+                       x_dev, tab_dev, col_dev, (int)K, (int)H, (int)W, (int)OW, (int)(OH * OW), (int)stride, (int)pad,
+                       make_fastdiv(OH * OW), make_fastdiv(OW));
     hipError_t e = hipGetLastError();
     rc = nbl_free(ctx, tab_dev);   // waits for the kernel
     if(e != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "launch of im2col_kernel failed: %s", hipGetErrorString(e));
