@@ -95,6 +95,7 @@ def oracle():
         lib.orc_perplexity.restype = C.c_float
         lib.orc_image_to_input.argtypes = [C.c_void_p, _u, _u, _u, _f32p, _u, _u]
         lib.orc_resize_linear_u8.argtypes = [C.c_void_p, _u, _u, _u, C.c_void_p, _u, _u]
+        lib.orc_linear_taps.argtypes = [_u, _u, C.c_int, C.c_void_p, C.c_void_p]
         pp = C.POINTER(_f32p)
         lib.orc_rnn_forward.argtypes = [_f32p, pp, pp, pp, pp, pp, _f32p, _u, _u, _u, _u, _u]
         lib.orc_topk_matches.argtypes = [_f32p, C.c_void_p, _u, _u, _u]
@@ -243,6 +244,14 @@ def image_to_input(img, dst_h, dst_w):
     out = np.empty((c, dst_h, dst_w), np.float32)
     oracle().orc_image_to_input(img.ctypes.data, h, w, c, _fp(out), dst_h, dst_w)
     return out
+
+
+def linear_taps(dst_n, src_n, clamp_weight):
+    """First source index and the two 11-bit weights of every destination pixel along one axis."""
+    ofs = np.empty(dst_n, np.int32)
+    w = np.empty((dst_n, 2), np.int16)
+    oracle().orc_linear_taps(dst_n, src_n, int(clamp_weight), ofs.ctypes.data, w.ctypes.data)
+    return ofs, w
 
 
 def resize_linear_u8(img, dst_h, dst_w):

@@ -393,13 +393,18 @@ void orc_softmax_forward(const float *x, float *y, unsigned rows, unsigned n) {
  * (resize.cpp: pixel-centre mapping fx = (dx + 0.5) * scale - 0.5; horizontal and vertical
  * weights as shorts scaled by 2048 with round-half-even; horizontal pass in int; vertical
  * pass ((b0 * (S0 >> 4)) >> 16) + ((b1 * (S1 >> 4)) >> 16) + 2) >> 2).  Pinned only by
- * mathematics: identity at equal size, constants stay constant, within one grey level of
- * exact bilinear interpolation (tests/test_oracle_math.py).  The byte -> float planes and
- * the plane swap are pinned bit for bit by their closed form.
+ * mathematics (tests/test_oracle_math.py): identity at equal size, constants stay constant,
+ * within one grey level of exact bilinear interpolation; tap tables equal to their rational
+ * closed form (source index and 11-bit weight of every destination pixel, from exact
+ * fractions); exact halving equal to the rounded 2x2 box mean that OpenCV itself substitutes
+ * for that ratio (INTER_AREA, same result by construction); exact doubling equal to the
+ * 1/4 : 3/4 stencil on ramps (no rounding occurs) and impulses.  The byte -> float planes
+ * and the plane swap are pinned bit for bit by their closed form.
  * ------------------------------------------------------------------------------------- */
 static int orc_round_half_even(double v) { return (int)nearbyint(v); }   /* default rounding mode */
 
-static void orc_linear_taps(unsigned dst_n, unsigned src_n, int clamp_weight, int *ofs, short *w) {
+/* Exported so that the tests can hold the table against its rational closed form. */
+void orc_linear_taps(unsigned dst_n, unsigned src_n, int clamp_weight, int *ofs, short *w) {
     const double scale = (double)src_n / (double)dst_n;
     for(unsigned d = 0; d < dst_n; d++) {
         float f = (float)((d + 0.5) * scale - 0.5);

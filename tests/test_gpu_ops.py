@@ -196,7 +196,7 @@ def test_activation_kernels(ctx, name):
 
 
 IMAGES = [(2, 13, 17, 3, 13, 17), (3, 40, 30, 3, 16, 12), (2, 31, 29, 3, 47, 18), (1, 8, 8, 3, 227, 227), (2, 64, 48, 1, 5, 5),
-          (1, 375, 500, 3, 224, 224)]
+          (1, 375, 500, 3, 224, 224), (2, 16, 20, 3, 8, 10), (1, 9, 12, 3, 18, 24), (1, 454, 454, 3, 227, 227)]
 
 
 @pytest.mark.parametrize("case", IMAGES)

@@ -224,3 +224,97 @@ def test_image_input_contract_closed_form_and_resize_bounds():
         assert np.abs(got - exact).mean() < 0.35
     gray = rng.integers(0, 256, (10, 12, 1), dtype=np.uint8)
     np.testing.assert_array_equal(ob.image_to_input(gray, 10, 12)[0], (gray[..., 0] / 255.0).astype(np.float32))
+
+
+def _exact_taps(dst_n, src_n, clamp_weight):
+    """Source index and weights of the pixel-centre mapping x = (d + 1/2) * src/dst - 1/2, from exact fractions."""
+    from fractions import Fraction
+    ofs, w, tie = [], [], []
+    for d in range(dst_n):
+        x = Fraction(2 * d + 1, 2) * Fraction(src_n, dst_n) - Fraction(1, 2)
+        s = x.numerator // x.denominator            # floor, also for negatives
+        f = x - s
+        if clamp_weight and s < 0:
+            s, f = 0, Fraction(0)
+        if clamp_weight and s >= src_n - 1:
+            s, f = src_n - 1, Fraction(0)
+        ofs.append(s)
+        w.append(f * 2048)
+        tie.append((f * 4096).denominator == 1 and (f * 2048).denominator != 1)
+    return ofs, w, tie
+
+
+@pytest.mark.parametrize("dst_n,src_n", [(8, 8), (16, 8), (8, 16), (24, 8), (8, 24), (32, 8), (227, 256), (224, 500), (224, 375), (47, 31),
+                                         (5, 64), (227, 8), (12, 30), (3, 2), (2, 3), (1, 7), (7, 1)])
+@pytest.mark.parametrize("clamp_weight", [0, 1])
+def test_resize_tap_table_against_rational_closed_form(dst_n, src_n, clamp_weight):
+    """The table of the resize restatement holds, per destination pixel, floor(x) and the weights (1 - f, f) * 2048 rounded
+    to the nearest integer, x being the exact rational pixel-centre coordinate; the two weights always add up to 2048.
+    A shifted mapping (corner alignment, a dropped half pixel), a swapped weight pair or a different scale fails here."""
+    ofs, w = ob.linear_taps(dst_n, src_n, clamp_weight)
+    want_ofs, want_w1, tie = _exact_taps(dst_n, src_n, clamp_weight)
+    np.testing.assert_array_equal(ofs, np.array(want_ofs, np.int32))
+    np.testing.assert_array_equal(w.astype(np.int64).sum(axis=1), np.full(dst_n, 2048))
+    for d in range(dst_n):
+        # the coordinate is held in float (as OpenCV holds it): its fraction is good to src_n * 2^-24
+        assert abs(float(w[d, 1]) - float(want_w1[d])) <= 0.5 + 2048 * max(src_n, 1) * 2.0 ** -23, (d, w[d], want_w1[d])
+        if want_w1[d].denominator == 1:
+            assert int(w[d, 1]) == int(want_w1[d])
+        if tie[d]:                                  # an exact half rounds to the even neighbour
+            assert int(w[d, 1]) % 2 == 0
+
+
+def test_resize_exact_halving_is_the_rounded_box_mean():
+    """At exactly half size every weight is 1024/2048 and the fixed-point passes lose nothing:
+    dst = (a + b + c + d + 2) >> 2 over each 2x2 block, the result OpenCV's own 2x2 area path gives for this ratio."""
+    rng = np.random.default_rng(11)
+    for (h, w, c) in [(8, 10, 3), (64, 48, 1), (454, 454, 3), (2, 2, 4)]:
+        src = rng.integers(0, 256, (h, w, c), dtype=np.uint8)
+        s = src.astype(np.int64)
+        want = (s[0::2, 0::2] + s[0::2, 1::2] + s[1::2, 0::2] + s[1::2, 1::2] + 2) >> 2
+        np.testing.assert_array_equal(ob.resize_linear_u8(src, h // 2, w // 2), want.astype(np.uint8))
+        ofs, wt = ob.linear_taps(w // 2, w, 1)
+        np.testing.assert_array_equal(ofs, 2 * np.arange(w // 2))
+        assert (wt == 1024).all()
+    extremes = np.zeros((4, 4, 1), np.uint8); extremes[:2] = 255
+    np.testing.assert_array_equal(ob.resize_linear_u8(extremes, 2, 2)[..., 0], [[255, 255], [0, 0]])
+
+
+def test_resize_exact_doubling_is_the_quarter_stencil():
+    """At exactly double size the taps are 1/4 : 3/4 (512 / 1536 of 2048), with the border pixel repeated.  On ramps
+    whose steps are multiples of 16 no intermediate is rounded, so the output is the stencil's exact value; an impulse
+    returns the separable response [1, 3, 3, 1] x [1, 3, 3, 1] / 16 with the scheme's truncations."""
+    ofs, wt = ob.linear_taps(16, 8, 1)
+    np.testing.assert_array_equal(ofs, [0, 0, 0, 1, 1, 2, 2, 3, 3, 4, 4, 5, 5, 6, 6, 7])
+    np.testing.assert_array_equal(wt[:, 1], [0] + [512, 1536] * 7 + [0])
+    ofs, wt = ob.linear_taps(16, 8, 0)                       # rows: weights stay, the row index is clipped later
+    np.testing.assert_array_equal(ofs, [-1] + [k // 2 for k in range(15)])
+    np.testing.assert_array_equal(wt[:, 1], [1536, 512] * 8)
+
+    def stencil(v):                                          # exact 1-D doubling of an integer sequence, times 4
+        p = np.concatenate([v[:1], v, v[-1:]]).astype(np.int64)
+        out = np.empty(2 * len(v), np.int64)
+        out[0::2] = p[:-2] + 3 * p[1:-1]
+        out[1::2] = 3 * p[1:-1] + p[2:]
+        return out
+    xs = 16 * np.arange(12)
+    ys = 16 * np.arange(9)
+    ramp = (xs[None, :] + ys[:, None])
+    ramp = np.where(ramp > 240, 480 - ramp, ramp).astype(np.uint8)      # a ridge, still piecewise linear in steps of 16
+    hor = np.stack([stencil(r) for r in ramp.astype(np.int64)])         # times 4
+    both = np.stack([stencil(col) for col in hor.T]).T                  # times 16
+    assert (both % 16 == 0).all()
+    np.testing.assert_array_equal(ob.resize_linear_u8(ramp[..., None], 18, 24)[..., 0], (both // 16).astype(np.uint8))
+
+    imp = np.zeros((6, 7, 1), np.uint8); imp[2, 3] = 255
+    got = ob.resize_linear_u8(imp, 12, 14)[..., 0].astype(np.int64)
+    k = np.array([1, 3, 3, 1])
+    exact = 255 * np.outer(k, k) / 16.0
+    blk = got[3:7, 5:9]
+    assert np.abs(blk - exact).max() < 1.0 and got.sum() == blk.sum()
+    np.testing.assert_array_equal(blk, blk.T)
+    np.testing.assert_array_equal(blk, blk[::-1, ::-1])
+    # the scheme itself on this block: horizontal sums 255 * {512, 1536}, >> 4, times the row weight, >> 16, + 2 >> 2
+    h4 = 255 * np.array([512, 1536, 1536, 512])
+    fixed = ((((np.array([512, 1536, 1536, 512])[:, None] * (h4[None, :] >> 4)) >> 16) + 2) >> 2)
+    np.testing.assert_array_equal(blk, fixed)
