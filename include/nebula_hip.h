@@ -115,6 +115,8 @@ int nbl_conv2d_plan_info(const nbl_conv_plan *plan, unsigned *OH, unsigned *OW, 
  * image staged in LDS: variant == nbl_conv2d_num_variants() names it (NBL_EINVAL for a plan that does not qualify;
  * it fuses no shortcut: nbl_conv2d_shortcut_fwd falls back to a tile shape). */
 int nbl_conv2d_plan_set_variant(nbl_conv_plan *plan, int variant);
+/* Name of a tile shape ("128x128", "64x64", ..., "strip" for index nbl_conv2d_num_variants()); NULL out of range. */
+const char *nbl_conv2d_variant_name(int variant);
 /* k-split of launches whose tile count leaves CUs idle in the last round: the tiles of that round are
  * cut into slices along C*k*k, one block each, and a second small kernel adds the slices in slice order
  * and applies the epilogue (the result does not depend on timing, but it differs in the last bits from

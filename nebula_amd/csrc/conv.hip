@@ -936,6 +936,10 @@ extern "C" {
 
 int nbl_conv2d_num_variants(void) { return NUM_VARIANTS; }
 
+const char *nbl_conv2d_variant_name(int variant) {
+    return variant == NUM_VARIANTS ? "strip" : variant >= 0 && variant < NUM_VARIANTS ? VARIANTS[variant].name : NULL;
+}
+
 int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
                     const float *scale_host, const float *mean_host, const float *var_host,
                     unsigned C, unsigned H, unsigned W, unsigned F,

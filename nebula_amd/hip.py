@@ -56,6 +56,7 @@ SIGNATURES = {
     "nbl_conv2d_plan_set_split": (C.c_int, [_vp, C.c_int]),
     "nbl_conv2d_plan_last_launch": (C.c_int, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "nbl_conv2d_num_variants": (C.c_int, []),
+    "nbl_conv2d_variant_name": (C.c_char_p, [C.c_int]),
     "nbl_im2col": (C.c_int, [_vp, _vp, _u, _u, _u, _u, _u, _u, _vp]),
     "nbl_fc_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_fc_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u]),

@@ -38,6 +38,8 @@ def test_no_device_is_reported_not_crashed():
     assert l.nbl_pool_out_dim(55, 2, 0) == 27 and l.nbl_pool_out_dim(112, 2, 0) == 56
     assert l.nbl_conv_out_dim(227, 11, 4, 0) == 55 and l.nbl_conv_out_dim(224, 7, 2, 3) == 112
     assert l.nbl_conv2d_num_variants() >= 1
+    assert l.nbl_conv2d_variant_name(l.nbl_conv2d_num_variants()) == b"strip" and l.nbl_conv2d_variant_name(-1) is None
+    assert l.nbl_conv2d_variant_name(0) == b"128x128"
 
 
 def test_layers_library_exports_and_reports_missing_device():
