@@ -473,6 +473,10 @@ __global__ void image_to_input_kernel(const unsigned char *__restrict__ src, flo
 }
 
 // Source index and the two weights of every destination coordinate along one axis.
+// At exactly half size every coordinate falls midway between two source pixels: both weights are 1024 of 2048, the
+// fixed-point passes then lose nothing and the result is (a + b + c + d + 2) >> 2 over each 2x2 block -- the same
+// bytes as the 2x2 area average that cv::resize substitutes for INTER_LINEAR at that ratio, so the case needs no
+// branch of its own.
 static void linear_taps(unsigned dst_n, unsigned src_n, bool clamp_weight, std::vector<int> &ofs, std::vector<int> &weights) {
     ofs.resize(dst_n); weights.resize(dst_n);
     const double scale = (double)src_n / (double)dst_n;
