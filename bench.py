@@ -63,7 +63,7 @@ def make_weights(layout, rng, dist, lstm_hidden=1024):
 def workload(name, batch):
     from nebula_amd import zoo
     table = {
-        "resnet50": (lambda b: zoo.resnet50_cfg(b, fuse_shortcut=True), 64, "normal", "he",
+        "resnet50": (lambda b: zoo.resnet50_cfg(b, fuse_shortcut=True, in_place=True), 64, "normal", "he",
                      "ResNet-50 (Nebula topology) fp32 forward, batch %d, 3x224x224 N(0,1)"),
         "alexnet": (zoo.alexnet_cfg, 128, "uniform", "he", "AlexNet fp32 forward, batch %d, 3x227x227 U[0,1)"),
         "vgg16": (zoo.vgg16_cfg, 32, "normal", "he", "VGG-16 fp32 forward, batch %d, 3x224x224 N(0,1)"),

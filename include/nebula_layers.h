@@ -72,6 +72,11 @@ int nbl_net_forward_timed(nbl_net *net, float *ms);
 /* device -> host copy of layer's output ([batch_size][output_size]).  A convolution fused with the [shortcut] behind
  * it (fuse_shortcut=1) has no buffer of its own: its output is the shortcut's (the sum, activated). */
 int nbl_net_layer_output(nbl_net *net, int layer, float *host, size_t count);
+/* Whose values nbl_net_layer_output(layer) returns after a pass: *writer = layer itself for a layer with a tensor of
+ * its own; the [shortcut] behind it for a fused convolution; with shortcut_in_place=1 the last shortcut that wrote its
+ * result over this layer's tensor (a ResNet stage then shares one tensor between its blocks and only the last block's
+ * output survives the pass). */
+int nbl_net_layer_output_writer(nbl_net *net, int layer, int *writer);
 /* The max-pool argmax table the reference's forward keeps for its backward pass (pooling_layer.cc:132,140):
  * flat offsets into the layer's input tensor.  Kept only when the [net] section says pool_index=1 (a key the
  * reference ignores); inference never reads the table, so by default it is not written. */

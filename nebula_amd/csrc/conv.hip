@@ -1230,6 +1230,17 @@ static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_
         if(p->tuned_batch != B) {
             // the search overwrites y with correct results several times; tiny problems are not worth it
             if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); p->tuned_slices = p->split_mode > 0 ? p->split_mode : 0; }
+            else if(rs && rs->res == y_dev) {
+                // in place: the search's many launches must not feed on their own output, so they write to a buffer
+                // of their own (the residual is only read) and the real launch below is the one that writes y
+                float *tmp = NULL;
+                int rc = nbl_malloc(ctx, (void**)&tmp, out_elems * sizeof(float));
+                if(rc != NBL_OK) return rc;
+                rc = conv_tune(ctx, p, x_dev, tmp, B, rs);
+                const int rc_free = nbl_free(ctx, tmp);       // waits for the search's launches
+                if(rc != NBL_OK) return rc;
+                if(rc_free != NBL_OK) return rc_free;
+            }
             else { int rc = conv_tune(ctx, p, x_dev, y_dev, B, rs); if(rc != NBL_OK) return rc; }
         }
         v = p->tuned_variant;
@@ -1252,7 +1263,10 @@ int nbl_conv2d_shortcut_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float
     NBL_REQUIRE(ctx, plan && x_dev && y_dev && conn_dev, "nbl_conv2d_shortcut_fwd: NULL argument");
     NBL_REQUIRE(ctx, conn_c && conn_h && conn_w, "nbl_conv2d_shortcut_fwd: zero dimension");
     NBL_REQUIRE(ctx, nbl_act_valid(post_act), "nbl_conv2d_shortcut_fwd: undefined activation type %d", post_act);
-    NBL_REQUIRE(ctx, y_dev != conn_dev, "nbl_conv2d_shortcut_fwd: y must not alias conn");
+    // Writing the result over the residual is sound when the two have the same shape: every element is then read and
+    // written by the same lane (also in the finishing kernel of a k-split launch), and nothing else reads conn.
+    NBL_REQUIRE(ctx, y_dev != conn_dev || (conn_c == plan->F && conn_h == plan->OH && conn_w == plan->OW),
+                "nbl_conv2d_shortcut_fwd: y may alias conn only when conn has the output's shape");
     if(plan->OW / conn_w > 1)
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: an up-sampling shortcut cannot be fused");
     if((size_t)B * conn_c * conn_h * conn_w >= (1ull << 31))

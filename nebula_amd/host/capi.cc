@@ -163,6 +163,20 @@ int nbl_net_layer_output(nbl_net *n, int i, float *host, size_t count) {
         nbl_check(n->net->ctx, nbl_d2h(n->net->ctx, host, l->output_data_dev, count * sizeof(float)), "nbl_d2h"));
 }
 
+int nbl_net_layer_output_writer(nbl_net *n, int i, int *writer) {
+    NBL_NET_TRY(
+        layer_t *l = layer_at(n, i);
+        if(!writer) throw std::runtime_error("Error: writer is NULL");
+        // the last layer with a kernel of its own whose output pointer is this layer's
+        *writer = i;
+        const std::vector<layer_t*> &layers = n->net->layers;
+        for(int j = i + 1; j < (int)layers.size(); j++) {
+            const layer_type_t t = layers[j]->layer_type;
+            if(t == DROPOUT_LAYER || t == COST_LAYER) continue;
+            if(layers[j]->output_data_dev && layers[j]->output_data_dev == l->output_data_dev) *writer = j;
+        });
+}
+
 int nbl_net_pool_index(nbl_net *n, int i, unsigned *host, size_t count) {
     NBL_NET_TRY(
         layer_t *l = layer_at(n, i);

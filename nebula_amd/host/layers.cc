@@ -346,7 +346,7 @@ void pooling_layer_t::_forward_() {
 
 // ---- shortcut --------------------------------------------------------------------------------------
 shortcut_layer_t::shortcut_layer_t(network_t *m_network, layer_t *m_prev_layer, layer_type_t m_layer_type) :
-    layer_t(m_network, m_prev_layer, m_layer_type), connection(NULL), fused(false), hops(0) {}
+    layer_t(m_network, m_prev_layer, m_layer_type), connection(NULL), fused(false), in_place(false), hops(0) {}
 
 shortcut_layer_t::~shortcut_layer_t() {}
 
@@ -371,6 +371,15 @@ void shortcut_layer_t::init(section_config_t m_section_config) {
     output_size = output_height * output_width * output_channel;
     input_size = output_size;
     alloc_output();
+}
+
+void shortcut_layer_t::write_over_connection() {
+    if(!fused || in_place || !connection || !prev_layer) return;
+    if(owns_output && output_data_dev && network->ctx) nbl_free(network->ctx, output_data_dev);
+    owns_output = false;
+    output_data_dev = connection->output_data_dev;
+    prev_layer->output_data_dev = output_data_dev;      // the fused convolution aliases this layer's tensor
+    in_place = true;
 }
 
 void shortcut_layer_t::_forward_() {

@@ -143,6 +143,10 @@ public:
     void _forward_();
     layer_t *connection;       // the layer `hops` back whose output is added
     bool fused;                // computed by the preceding convolution's epilogue; _forward_() does nothing
+    // Give up this layer's own buffer and write the result over the connection's tensor (same shape, fused only):
+    // this layer's output pointer, and the fused convolution's, become aliases of the connection's.
+    void write_over_connection();
+    bool in_place;
 private:
     unsigned hops;
 };

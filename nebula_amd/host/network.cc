@@ -66,7 +66,7 @@ void network_t::store_weight(const std::string m_output_weight) {
 
 // ---- inference_net_t -------------------------------------------------------------------------------
 inference_net_t::inference_net_t(int device, unsigned m_batch_override) :
-    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), last_step_only(false), fuse_shortcut(false), use_graph(false),
+    cumulative_cost(0.0f), rows_seen(0), topk_matches(0), last_step_only(false), fuse_shortcut(false), shortcut_in_place(false), use_graph(false),
     first_after_lstm(-1), batch_override(m_batch_override), is_recurrent(false), image_staging_dev(NULL),
     tokens_dev(NULL), labels_dev(NULL), cost_dev(NULL), image_staging_bytes(0),
     graph_exec(NULL), graph_key(0), warm_key(0), graph_epoch(1), graph_unusable(false) {
@@ -125,6 +125,7 @@ void inference_net_t::build(config_t &config) {
             sc.get_setting("channels", &input_channel);
             sc.get_setting("batch", &batch_size);
             sc.get_setting("fuse_shortcut", &fuse_shortcut);
+            sc.get_setting("shortcut_in_place", &shortcut_in_place);
             sc.get_setting("hip_graph", &use_graph);
             sc.get_setting("pool_index", &pool_index);
             if(sc.exists("conv_split")) { unsigned v = 0; sc.get_setting("conv_split", &v); conv_split = v ? 1 : 0; }
@@ -175,6 +176,38 @@ void inference_net_t::build(config_t &config) {
                 if(!read_elsewhere)
                     static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
             }
+    if(fuse_shortcut && shortcut_in_place) {
+        // The layer whose kernel really writes the tensor a layer's output pointer refers to: dropout and cost layers
+        // alias their producer, a fused convolution writes its shortcut's tensor.
+        std::vector<int> producer(num_layers);
+        for(unsigned i = 0; i < num_layers; i++) {
+            producer[i] = (int)i;
+            if((layers[i]->layer_type == DROPOUT_LAYER || layers[i]->layer_type == COST_LAYER) && i > 0) producer[i] = producer[i - 1];
+        }
+        auto index_of = [&](const layer_t *l) { for(unsigned i = 0; i < num_layers; i++) if(layers[i] == l) return (int)i; return -1; };
+        for(unsigned i = 1; i < num_layers; i++) {
+            if(layers[i]->layer_type != SHORTCUT_LAYER) continue;
+            shortcut_layer_t *sc = static_cast<shortcut_layer_t*>(layers[i]);
+            if(!sc->fused) continue;
+            const int conn = index_of(sc->connection);
+            if(conn < 0) continue;
+            const layer_t *c = layers[conn];
+            if(c->output_channel != sc->output_channel || c->output_height != sc->output_height || c->output_width != sc->output_width) continue;
+            const int tensor = producer[conn];
+            // every other reader of that tensor must run before the fused convolution (layer i - 1) starts writing
+            bool safe = true;
+            for(unsigned j = 0; j < num_layers && safe; j++) {
+                if(j == i) continue;
+                const bool reads_as_input = j > 0 && producer[j - 1] == tensor && producer[j] == (int)j;
+                const bool reads_as_connection = layers[j]->layer_type == SHORTCUT_LAYER &&
+                                                 index_of(static_cast<shortcut_layer_t*>(layers[j])->connection) >= 0 &&
+                                                 producer[index_of(static_cast<shortcut_layer_t*>(layers[j])->connection)] == tensor;
+                if((reads_as_input || reads_as_connection) && j >= i - 1) safe = false;
+            }
+            if(layers[tensor] == output_layer) safe = false;
+            if(safe) sc->write_over_connection();
+        }
+    }
     for(unsigned i = 0; i < num_layers; i++)
         if(layers[i]->layer_type == LSTM_LAYER || layers[i]->layer_type == RNN_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;
 }

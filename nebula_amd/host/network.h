@@ -117,6 +117,13 @@ public:
     // [shortcut] computes the residual add and the shortcut's activation in its own epilogue.  Same float
     // operations in the same order; the convolution's pre-shortcut output is then never materialised.
     bool fuse_shortcut;
+    // [net] key `shortcut_in_place=1` (with fuse_shortcut; a key the reference ignores): a fused shortcut whose
+    // connection has the output's shape writes its result over the connection's tensor instead of into a buffer of
+    // its own, wherever every other reader of that tensor runs before the fused convolution.  Each element is read
+    // and written by the same lane, so the values are the same; what changes is that the connection layer's output
+    // no longer exists after the pass (nbl_net_layer_output of it returns the shortcut's tensor) and that the
+    // memory system sees one address stream for residual and result (a 64x256x56x56 residual layer: 106 -> 84 us).
+    bool shortcut_in_place;
     // [net] key `hip_graph=1` (a key the reference ignores): forward() records the launches of one pass into a
     // HIP graph and replays it from then on, so a pass costs one launch on the host instead of one per kernel
     // (recurrent nets launch a kernel per layer and time step).  The first pass of a configuration runs

@@ -34,6 +34,7 @@ SIGNATURES = {
     "nbl_net_sync": (C.c_int, [_vp]),
     "nbl_net_forward_timed": (C.c_int, [_vp, C.POINTER(C.c_float)]),
     "nbl_net_layer_output": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
+    "nbl_net_layer_output_writer": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_int)]),
     "nbl_net_pool_index": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
     "nbl_net_conv_last_launch": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "nbl_net_conv_pin_launch": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int]),
@@ -174,6 +175,12 @@ class Network:
         out = np.empty(info["output_size"] * self.batch_size, np.float32)
         self._check(lib().nbl_net_layer_output(self.h, i, out.ctypes.data, out.size))
         return out
+
+    def output_writer(self, i):
+        """Index of the layer whose values output(i) returns (i itself unless the tensor is shared or overwritten)."""
+        w = C.c_int()
+        self._check(lib().nbl_net_layer_output_writer(self.h, i, C.byref(w)))
+        return w.value
 
     def pool_index(self, i):
         info = self.layer_info(i)

@@ -56,10 +56,12 @@ def vgg16_cfg(batch=32):
     return s
 
 
-def resnet50_cfg(batch=64, activation="relu", fuse_shortcut=False):
+def resnet50_cfg(batch=64, activation="relu", fuse_shortcut=False, in_place=False):
     """fuse_shortcut: let each block's last convolution add the residual in its epilogue (a [net] key the
-    reference ignores; results are bit-identical to the unfused network)."""
-    s = _net(batch, 224, 224, 3, "fuse_shortcut=1\n" if fuse_shortcut else "")
+    reference ignores; results are bit-identical to the unfused network).  in_place: a fused shortcut whose
+    connection has the output's shape writes its result over the connection's tensor (same values; the connection
+    layer's own output is gone after the pass)."""
+    s = _net(batch, 224, 224, 3, ("fuse_shortcut=1\n" if fuse_shortcut else "") + ("shortcut_in_place=1\n" if in_place else ""))
     s += _conv(64, 7, 2, 3, activation, bn=True) + _pool("maxpool", 3, 2, 0)
     for stage, (width, blocks) in enumerate(((64, 3), (128, 4), (256, 6), (512, 3))):
         for block in range(blocks):

@@ -45,8 +45,14 @@ def oracle_forward(cfg, blob, x):
 def bench_cfg(batch):
     """The cfg text bench.py's default workload builds."""
     cfg, b, _, _, _ = bench.workload("resnet50", batch)
-    assert b == batch and "fuse_shortcut=1" in cfg
+    assert b == batch and "fuse_shortcut=1" in cfg and "shortcut_in_place=1" in cfg
     return cfg
+
+
+def survives(net, i):
+    """True when output(i) still holds layer i's own values after a pass (not a fused convolution, and not a tensor a
+    later in-place shortcut wrote over)."""
+    return net.output_writer(i) == i
 
 
 def test_benched_resnet50_cfg_against_oracle_layer_by_layer():
@@ -59,16 +65,26 @@ def test_benched_resnet50_cfg_against_oracle_layer_by_layer():
     net.set_input(x)
     net.forward()
     kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
-    fused = 0
+    fused = overwritten = 0
     for i, k in enumerate(kinds):
         if k in ("cost_layer", "dropout_layer"):
             continue
         if k == "convolutional_layer" and kinds[i + 1] == "shortcut_layer":
             fused += 1          # no buffer of its own: its output IS the shortcut's, compared at the next index
+            assert net.output_writer(i) >= i + 1
+            continue
+        if not survives(net, i):
+            # a same-shape shortcut of the next block wrote its result over this one's tensor; what it holds now is
+            # that later layer's output, which is compared at its own index
+            overwritten += 1
+            w = net.output_writer(i)
+            assert kinds[i] == "shortcut_layer" and kinds[w] == "shortcut_layer" and w > i
+            np.testing.assert_array_equal(bits(net.output(i)), bits(net.output(w)))
             continue
         r = rel(net.output(i), want[i].ravel())
         assert r <= TOL, (i, k, r)
     assert fused == 16
+    assert overwritten == 12        # 16 blocks, 4 stages: the last block's output of every stage survives
     last = max(i for i, k in enumerate(kinds) if k == "connected_layer")
     np.testing.assert_array_equal(net.output(last).reshape(2, -1).argmax(1), want[last].reshape(2, -1).argmax(1))
     net.close()
@@ -102,6 +118,8 @@ def test_benched_resnet50_batch64_fused_searched_split():
     for i, k in enumerate(kinds):
         if k in ("cost_layer", "dropout_layer") or (k == "convolutional_layer" and kinds[i + 1] == "shortcut_layer"):
             continue
+        if not survives(net64, i):
+            continue
         r = rel(net64.output(i), plain.output(i))
         worst = max(worst, r)
         assert r <= TOL, (i, k, r)
@@ -128,6 +146,20 @@ def test_benched_resnet50_batch64_fused_searched_split():
     assert [pinned.conv_last_launch(i) for i in convs] == launches
     np.testing.assert_array_equal(bits(pinned.output(last)), bits(net64.output(last)))
     pinned.close()
+
+    # (4) the same launches with every shortcut writing into a buffer of its own: every element is read and written
+    # by the same lane either way, so the surviving tensors agree bit for bit
+    own_cfg = bench_cfg(64).replace("shortcut_in_place=1\n", "")
+    own, _ = build(own_cfg)
+    for i, (v, g) in zip(convs, launches):
+        own.conv_pin_launch(i, v, g if g > 1 else 0)
+    own.set_input(x)
+    own.forward()
+    assert all(own.output_writer(i) == i for i, k in enumerate(kinds) if k == "shortcut_layer")
+    for i, k in enumerate(kinds):
+        if k in ("shortcut_layer", "connected_layer", "avgpool_layer") and survives(net64, i):
+            np.testing.assert_array_equal(bits(own.output(i)), bits(net64.output(i)), err_msg="layer %d" % i)
+    own.close()
     net64.close()
 
 
@@ -372,3 +404,51 @@ def test_fusion_is_skipped_when_a_later_shortcut_reads_the_convolution():
     # layer 1 (second convolution) is read by the last shortcut: it keeps its own output in the fused network too
     for i in (0, 1, 2, 4):
         np.testing.assert_array_equal(bits(outs[0][i]), bits(outs[1][i]), err_msg="layer %d" % i)
+
+
+@pytest.mark.parametrize("shape", [(64, 56, 256), (256, 14, 1024), (512, 7, 2048), (96, 10, 80)])
+def test_fused_residual_written_in_place(shape):
+    """nbl_conv2d_shortcut_fwd with y == conn (same shape): the result replaces the residual and equals, bit for bit, what
+    the same launch writes into a separate buffer -- for every tile shape, split and unsplit, and through the tile search
+    (whose trial launches must not feed on their own output)."""
+    from nebula_amd import hip
+    Cc, HW, F = shape
+    B = 4
+    print("CASE in-place fused residual", shape, flush=True)
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal((B, Cc, HW, HW)).astype(np.float32)
+    w = (rng.standard_normal((F, Cc, 1, 1)) * np.sqrt(2.0 / Cc)).astype(np.float32)
+    bias = (rng.standard_normal(F) * 0.1).astype(np.float32)
+    conn = rng.standard_normal((B, F, HW, HW)).astype(np.float32)
+    assert ob.use_openblas(threads=16)
+    try:
+        want = ob.shortcut_forward(ob.conv_forward(x, w, bias, None, 1, 0, "linear"), conn, "relu")
+    finally:
+        ob.use_custom_gemm()
+        ob.set_threads(1)
+    with hip.Ctx(0) as ctx:
+        plan = ctx.conv_pack(w, bias, None, H=HW, W=HW, stride=1, pad=0, act="linear")
+        dx = ctx.array(x)
+        for v in list(range(hip.lib().nbl_conv2d_num_variants())) + [-1]:
+            for split in ((0, 1, 5) if v >= 0 else (-1,)):
+                print("   variant", v, "split", split, flush=True)
+                plan.set_variant(v)
+                plan.set_split(split)
+                dconn, dy = ctx.array(conn), ctx.empty(conn.shape)
+                if v < 0:
+                    in_place = plan.with_shortcut(dx, dconn, "relu", out=dconn).numpy()       # the search runs here
+                    launch = plan.last_launch()
+                    dconn.upload(conn)
+                    separate = plan.with_shortcut(dx, dconn, "relu", out=dy).numpy()
+                    assert plan.last_launch() == launch
+                else:
+                    separate = plan.with_shortcut(dx, dconn, "relu", out=dy).numpy()
+                    np.testing.assert_array_equal(bits(dconn.numpy()), bits(conn))              # residual untouched
+                    in_place = plan.with_shortcut(dx, dconn, "relu", out=dconn).numpy()
+                assert rel(separate, want) <= TOL, (shape, v, split)
+                np.testing.assert_array_equal(bits(in_place), bits(separate), err_msg="%r variant %d split %d" % (shape, v, split))
+                dconn.free(); dy.free()
+        # a connection of another shape cannot be the output
+        narrow = ctx.array(conn[:, : F // 2])
+        rc = hip.lib().nbl_conv2d_shortcut_fwd(ctx.h, plan.p, dx.ptr, narrow.ptr, F // 2, HW, HW, narrow.ptr, B, hip.ACT["relu"])
+        assert rc != 0 and b"alias" in hip.lib().nbl_last_error(ctx.h)
