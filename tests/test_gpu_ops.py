@@ -241,7 +241,11 @@ def test_activation_rejects_undefined(ctx):
 
 POOL = [(2, 3, 12, 12, 3, 2, 1), (2, 2, 13, 11, 3, 2, 0), (1, 4, 8, 8, 2, 2, 0), (2, 5, 7, 7, 7, 7, 0),
         (1, 2, 9, 9, 2, 1, 1), (1, 1, 6, 6, 5, 3, 2), (3, 16, 55, 55, 3, 2, 0), (2, 8, 112, 112, 3, 2, 0), (2, 4, 28, 28, 2, 2, 0),
-        (1, 3, 16, 12, 3, 2, 0), (2, 2, 14, 14, 7, 7, 0), (1, 2, 21, 21, 7, 2, 3)]
+        (1, 3, 16, 12, 3, 2, 0), (2, 2, 14, 14, 7, 7, 0), (1, 2, 21, 21, 7, 2, 3),
+        # rows that are not whole 16-byte pieces (AlexNet's maps): odd plane counts, padding, stride 1, a 5x5 window, a
+        # non-square plane, and AlexNet's first pool at its full size
+        (5, 23, 27, 27, 3, 2, 0), (16, 40, 13, 13, 3, 2, 0), (4, 24, 27, 27, 3, 2, 1), (2, 12, 55, 55, 2, 1, 1),
+        (3, 24, 31, 31, 5, 3, 2), (4, 10, 45, 39, 3, 2, 0), (128, 96, 55, 55, 3, 2, 0)]
 
 
 @pytest.mark.parametrize("geom", POOL)
