@@ -245,6 +245,11 @@ def memory_bound_kernels(args):
     timed("maxpool 2x2/2 32x64x224x224 (no argmax table)", 4 * (x.size + y.size),
           lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, None, 32, 64, 224, 224, 2, 2, 0, hip.POOL_MAX)))
     x.free(); y.free()
+    # AlexNet's first max-pool 3x3 / 2 at batch 128: rows of 55 floats (not whole 16-byte pieces)
+    x = rand((128, 96, 55, 55)); y = ctx.empty((128, 96, 27, 27))
+    timed("maxpool 3x3/2 128x96x55x55 (no argmax table)", 4 * (x.size + y.size),
+          lambda: ctx.check(l.nbl_pool_fwd(ctx.h, x.ptr, y.ptr, None, 128, 96, 55, 55, 3, 2, 0, hip.POOL_MAX)))
+    x.free(); y.free()
     # ResNet-50's closing 7x7 average pool
     x = rand((64, 2048, 7, 7)); y = ctx.empty((64, 2048))
     timed("avgpool 7x7 64x2048x7x7", 4 * (x.size + y.size),

@@ -74,6 +74,42 @@ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *_
     }
 }
 
+// A KS x KS window whose taps all lie inside the image (no padding, and the last window ends at or before the last row
+// and column: AlexNet's 3x3/2 pools on 55, 27 and 13 wide maps), any row length: a window row is KS adjacent floats,
+// fetched with ONE load of KS dwords at 4-byte alignment instead of KS loads (the address unit works per instruction,
+// and the general kernel's nine 4-byte loads per output held it to 40 % of the memory rate on these maps).
+template<int KS> struct __attribute__((packed, aligned(4))) WindowRow { float v[KS]; };
+template<bool IS_MAX, bool WRITE_INDEX, int KS>
+__global__ __launch_bounds__(256)
+void pool_inside_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
+                        unsigned total, int H, int W, int OH, int OW, int stride) {
+    const unsigned o = blockIdx.x * blockDim.x + threadIdx.x;
+    if(o >= total) return;
+    const unsigned ow = o % OW, t = o / OW, oh = t % OH, plane = t / OH;
+    const unsigned at0 = plane * (unsigned)(H * W) + oh * (unsigned)(stride * W) + ow * (unsigned)stride;
+    WindowRow<KS> rows[KS];
+    #pragma unroll
+    for(int i = 0; i < KS; i++) rows[i] = *reinterpret_cast<const WindowRow<KS>*>(x + at0 + i * W);
+    float best = -1e8f, acc = 0.0f;
+    unsigned best_at = 0xffffffffu;
+    #pragma unroll
+    for(int i = 0; i < KS; i++)
+        #pragma unroll
+        for(int j = 0; j < KS; j++) {
+            if(IS_MAX) {
+                if(rows[i].v[j] > best) { best = rows[i].v[j]; best_at = at0 + (unsigned)(i * W + j); }
+            } else {
+                acc += rows[i].v[j];
+            }
+        }
+    if(IS_MAX) {
+        y[o] = best;
+        if(WRITE_INDEX) index[o] = best_at;
+    } else {
+        y[o] = acc / (float)(KS * KS);
+    }
+}
+
 // Stride 2, no padding, image width a multiple of 4: a lane produces two adjacent outputs from one
 // 16-byte load per window row (plus one scalar for the fifth column of a 3-wide window), so the
 // lanes of a wave read whole rows contiguously.  Same scan order, sentinel and tie rule as above.
@@ -584,6 +620,21 @@ int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index
         return NBL_OK;
     }
     dim3 grid((unsigned)nbl_div_up_sz(total, 256)), block(256);
+    // every tap of every window inside the image: one load per window row
+    if(pad == 0 && (ksize == 2 || ksize == 3) && (OH - 1) * stride + ksize <= H && (OW - 1) * stride + ksize <= W) {
+#define NBL_INSIDE_LAUNCH(IS_MAX, WI, KS) \
+        hipLaunchKernelGGL((pool_inside_kernel<IS_MAX, WI, KS>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev, \
+                           (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)stride)
+        if(mode == NBL_POOL_MAX) {
+            if(index_dev) { if(ksize == 2) NBL_INSIDE_LAUNCH(true, true, 2); else NBL_INSIDE_LAUNCH(true, true, 3); }
+            else          { if(ksize == 2) NBL_INSIDE_LAUNCH(true, false, 2); else NBL_INSIDE_LAUNCH(true, false, 3); }
+        } else {
+            if(ksize == 2) NBL_INSIDE_LAUNCH(false, false, 2); else NBL_INSIDE_LAUNCH(false, false, 3);
+        }
+#undef NBL_INSIDE_LAUNCH
+        NBL_LAUNCH_CHECK(ctx, "pool_inside_kernel");
+        return NBL_OK;
+    }
 #define NBL_POOL_LAUNCH(IS_MAX, WI, KS) \
     hipLaunchKernelGGL((pool_kernel<IS_MAX, WI, KS>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev, \
                        (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)ksize, (int)stride, (int)pad)
