@@ -91,7 +91,7 @@ int nbl_sync(nbl_ctx *ctx);
  * nbl_conv2d_fwd replaces convolutional_layer_t::_forward_() (models/layers/convolutional_layer.cu:11-84;
  * CPU twin convolutional_layer.cc:365-409): per-image _im2col_ + cublasSgemm, _forward_batchnorm_,
  * _forward_bias_, _activate_ become one kernel.  x_dev [B][C][H][W] -> y_dev [B][F][OH][OW],
- * OH = (H + 2*pad - k)/stride + 1. */
+ * OH = (H + 2*pad - k)/stride + 1.  y_dev must not overlap x_dev (NBL_EINVAL). */
 int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
                     const float *scale_host, const float *mean_host, const float *var_host,
                     unsigned C, unsigned H, unsigned W, unsigned F,

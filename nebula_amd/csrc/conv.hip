@@ -1250,10 +1250,20 @@ static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_
     return conv_launch(ctx, p, x_dev, y_dev, B, v, slices, rs);
 }
 
+// [a, a + a_bytes) and [b, b + b_bytes) share a byte
+static bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
+    const size_t pa = (size_t)a, pb = (size_t)b;
+    return pa < pb + b_bytes && pb < pa + a_bytes;
+}
+
 int nbl_conv2d_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B) {
     if(!ctx) return NBL_EINVAL;
     NBL_REQUIRE(ctx, plan && x_dev && y_dev, "nbl_conv2d_fwd: NULL argument");
     if(B == 0) return NBL_OK;
+    // blocks read whole neighbourhoods of x while others write y
+    NBL_REQUIRE(ctx, !ranges_overlap(x_dev, (size_t)B * plan->C * plan->H * plan->W * sizeof(float),
+                                     y_dev, (size_t)B * plan->F * plan->OH * plan->OW * sizeof(float)),
+                "nbl_conv2d_fwd: y must not overlap x");
     return conv_forward(ctx, plan, x_dev, y_dev, B, NULL);
 }
 
@@ -1265,8 +1275,15 @@ int nbl_conv2d_shortcut_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float
     NBL_REQUIRE(ctx, nbl_act_valid(post_act), "nbl_conv2d_shortcut_fwd: undefined activation type %d", post_act);
     // Writing the result over the residual is sound when the two have the same shape: every element is then read and
     // written by the same lane (also in the finishing kernel of a k-split launch), and nothing else reads conn.
-    NBL_REQUIRE(ctx, y_dev != conn_dev || (conn_c == plan->F && conn_h == plan->OH && conn_w == plan->OW),
-                "nbl_conv2d_shortcut_fwd: y may alias conn only when conn has the output's shape");
+    const size_t y_bytes = (size_t)B * plan->F * plan->OH * plan->OW * sizeof(float);
+    if(y_dev == conn_dev)
+        NBL_REQUIRE(ctx, conn_c == plan->F && conn_h == plan->OH && conn_w == plan->OW,
+                    "nbl_conv2d_shortcut_fwd: y may alias conn only when conn has the output's shape");
+    else
+        NBL_REQUIRE(ctx, !ranges_overlap(conn_dev, (size_t)B * conn_c * conn_h * conn_w * sizeof(float), y_dev, y_bytes),
+                    "nbl_conv2d_shortcut_fwd: y may alias conn only as a whole (same address, same shape)");
+    NBL_REQUIRE(ctx, !ranges_overlap(x_dev, (size_t)B * plan->C * plan->H * plan->W * sizeof(float), y_dev, y_bytes),
+                "nbl_conv2d_shortcut_fwd: y must not overlap x");
     if(plan->OW / conn_w > 1)
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: an up-sampling shortcut cannot be fused");
     if((size_t)B * conn_c * conn_h * conn_w >= (1ull << 31))

@@ -524,6 +524,18 @@ def test_error_paths(ctx):
     # zero batch is a no-op, not an error
     plan = ctx.conv_pack(w, b, None, H=8, W=8, stride=1, pad=1, act="relu")
     assert l.nbl_conv2d_fwd(ctx.h, plan.p, d.ptr, d.ptr, 0) == 0
+    # a convolution reads whole neighbourhoods while other blocks write: output and input must not share memory, and the
+    # residual of a fused shortcut may be the output only as a whole
+    big = ctx.empty((4 * 2 * 8 * 8,))
+    assert l.nbl_conv2d_fwd(ctx.h, plan.p, big.ptr, big.ptr, 1) == -1 and b"overlap" in l.nbl_last_error(ctx.h)
+    assert l.nbl_conv2d_fwd(ctx.h, plan.p, big.ptr, big.ptr + 64, 1) == -1 and b"overlap" in l.nbl_last_error(ctx.h)
+    assert l.nbl_conv2d_fwd(ctx.h, plan.p, big.ptr, big.ptr + 4 * 2 * 8 * 8, 1) == 0                     # side by side is fine
+    y1 = ctx.empty((4 * 2 * 8 * 8,))
+    assert l.nbl_conv2d_shortcut_fwd(ctx.h, plan.p, big.ptr, y1.ptr, 2, 8, 8, y1.ptr + 16, 1, hip.ACT["relu"]) == -1
+    assert b"alias" in l.nbl_last_error(ctx.h)
+    assert l.nbl_conv2d_shortcut_fwd(ctx.h, plan.p, big.ptr, y1.ptr, 2, 8, 8, big.ptr, 1, hip.ACT["relu"]) == -1
+    assert b"overlap" in l.nbl_last_error(ctx.h)
+    assert l.nbl_conv2d_shortcut_fwd(ctx.h, plan.p, big.ptr, y1.ptr, 2, 8, 8, y1.ptr, 1, hip.ACT["relu"]) == 0   # in place
     # k-split modes: -1 (measured), 0, 1 and a slice count of 2..8
     assert l.nbl_conv2d_plan_set_split(plan.p, 9) != 0 and l.nbl_conv2d_plan_set_split(plan.p, -2) != 0
     assert l.nbl_conv2d_plan_set_split(plan.p, 8) == 0 and l.nbl_conv2d_plan_set_split(plan.p, -1) == 0
