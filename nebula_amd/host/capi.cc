@@ -167,13 +167,15 @@ int nbl_net_layer_output_writer(nbl_net *n, int i, int *writer) {
     NBL_NET_TRY(
         layer_t *l = layer_at(n, i);
         if(!writer) throw std::runtime_error("Error: writer is NULL");
-        // the last layer with a kernel of its own whose output pointer is this layer's
+        // the last layer with a kernel of its own that writes the tensor this layer's output pointer refers to
+        (void)l;
         *writer = i;
         const std::vector<layer_t*> &layers = n->net->layers;
-        for(int j = i + 1; j < (int)layers.size(); j++) {
+        const std::vector<int> &tensor = n->net->output_tensor;
+        for(int j = i + 1; j < (int)layers.size() && j < (int)tensor.size(); j++) {
             const layer_type_t t = layers[j]->layer_type;
             if(t == DROPOUT_LAYER || t == COST_LAYER) continue;
-            if(layers[j]->output_data_dev && layers[j]->output_data_dev == l->output_data_dev) *writer = j;
+            if(tensor[j] == tensor[i]) *writer = j;
         });
 }
 

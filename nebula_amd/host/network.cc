@@ -161,6 +161,14 @@ void inference_net_t::build(config_t &config) {
     }
     num_layers = (unsigned)layers.size();
     if(!output_layer && !layers.empty()) output_layer = layers.back();
+    // The layer whose kernel writes the tensor a layer's output pointer refers to, before any fusion: dropout and cost
+    // layers alias their producer.  (Indices, not pointers: a dry-run network has no buffers to compare.)
+    std::vector<int> producer(num_layers);
+    for(unsigned i = 0; i < num_layers; i++) {
+        producer[i] = (int)i;
+        if((layers[i]->layer_type == DROPOUT_LAYER || layers[i]->layer_type == COST_LAYER) && i > 0) producer[i] = producer[i - 1];
+    }
+    auto index_of = [&](const layer_t *l) { for(unsigned i = 0; i < num_layers; i++) if(layers[i] == l) return (int)i; return -1; };
     if(fuse_shortcut)
         for(unsigned i = 1; i < num_layers; i++)
             if(layers[i]->layer_type == SHORTCUT_LAYER && layers[i - 1]->layer_type == CONVOLUTIONAL_LAYER) {
@@ -170,21 +178,13 @@ void inference_net_t::build(config_t &config) {
                 bool read_elsewhere = false;
                 for(unsigned j = i + 1; j < num_layers && !read_elsewhere; j++)
                     if(layers[j]->layer_type == SHORTCUT_LAYER) {
-                        const layer_t *conn = static_cast<shortcut_layer_t*>(layers[j])->connection;
-                        read_elsewhere = conn == layers[i - 1] || (conn && conn->output_data_dev == layers[i - 1]->output_data_dev);
+                        const int conn = index_of(static_cast<shortcut_layer_t*>(layers[j])->connection);
+                        read_elsewhere = conn >= 0 && producer[conn] == (int)i - 1;
                     }
                 if(!read_elsewhere)
                     static_cast<convolutional_layer_t*>(layers[i - 1])->fuse_with(static_cast<shortcut_layer_t*>(layers[i]));
             }
     if(fuse_shortcut && shortcut_in_place) {
-        // The layer whose kernel really writes the tensor a layer's output pointer refers to: dropout and cost layers
-        // alias their producer, a fused convolution writes its shortcut's tensor.
-        std::vector<int> producer(num_layers);
-        for(unsigned i = 0; i < num_layers; i++) {
-            producer[i] = (int)i;
-            if((layers[i]->layer_type == DROPOUT_LAYER || layers[i]->layer_type == COST_LAYER) && i > 0) producer[i] = producer[i - 1];
-        }
-        auto index_of = [&](const layer_t *l) { for(unsigned i = 0; i < num_layers; i++) if(layers[i] == l) return (int)i; return -1; };
         for(unsigned i = 1; i < num_layers; i++) {
             if(layers[i]->layer_type != SHORTCUT_LAYER) continue;
             shortcut_layer_t *sc = static_cast<shortcut_layer_t*>(layers[i]);
@@ -207,6 +207,20 @@ void inference_net_t::build(config_t &config) {
             if(layers[tensor] == output_layer) safe = false;
             if(safe) sc->write_over_connection();
         }
+    }
+    // Which tensor every layer's output pointer refers to (the index of the layer that owns it): dropout and cost layers
+    // share their producer's, a fused convolution its shortcut's, an in-place shortcut its connection's.
+    output_tensor.assign(num_layers, 0);
+    for(unsigned i = 0; i < num_layers; i++) {
+        int t = (int)i;
+        if((layers[i]->layer_type == DROPOUT_LAYER || layers[i]->layer_type == COST_LAYER) && i > 0) t = output_tensor[i - 1];
+        if(layers[i]->layer_type == SHORTCUT_LAYER) {
+            const shortcut_layer_t *sc = static_cast<const shortcut_layer_t*>(layers[i]);
+            if(sc->in_place)
+                for(unsigned j = 0; j < i; j++) if(layers[j] == sc->connection) t = output_tensor[j];
+            if(sc->fused && i > 0) output_tensor[i - 1] = t;
+        }
+        output_tensor[i] = t;
     }
     for(unsigned i = 0; i < num_layers; i++)
         if(layers[i]->layer_type == LSTM_LAYER || layers[i]->layer_type == RNN_LAYER) first_after_lstm = i + 1 < num_layers ? (int)i + 1 : -1;

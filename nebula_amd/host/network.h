@@ -68,6 +68,7 @@ public:
     void store_weight(const std::string m_output_weight);
 
     std::vector<layer_t*> layers;
+    std::vector<int> output_tensor;      // per layer: index of the layer that owns the tensor its output pointer refers to
     layer_t *input_layer, *output_layer;
     unsigned num_layers;
 

@@ -26,12 +26,13 @@ def small_recurrent(kind, last_step_only=False):
     return zoo.rnn_cfg(batch=8, time_steps=5, input_size=96, hidden=64, layers=3, last_step_only=last_step_only), (5, 8, 96)
 
 
-CASES = ["mini_resnet", "mini_resnet_fused", "lstm", "lstm_last_step", "rnn", "dbn_like"]
+CASES = ["mini_resnet", "mini_resnet_fused", "mini_resnet_fused_in_place", "lstm", "lstm_last_step", "rnn", "dbn_like"]
 
 
 def build_case(name, rng):
     if name.startswith("mini_resnet"):
-        cfg = MINI_RESNET.replace("[net]\n", "[net]\nfuse_shortcut=1\n", 1) if name.endswith("fused") else MINI_RESNET
+        keys = "fuse_shortcut=1\nshortcut_in_place=1\n" if name.endswith("in_place") else "fuse_shortcut=1\n" if name.endswith("fused") else ""
+        cfg = MINI_RESNET.replace("[net]\n", "[net]\n" + keys, 1)
         shape = (4, 3, 32, 32)
     elif name.startswith("lstm"):
         cfg, shape = small_recurrent("lstm", name.endswith("last_step"))

@@ -377,3 +377,54 @@ def test_image_driver_topk_count(golden_dir):
         for k in (1, 2):
             total += ob.topk_matches(probs, labels, k)
             assert net.accumulate_topk(labels, k) == total
+
+
+def test_in_place_shortcuts_on_golden_resnet(golden_dir):
+    """shortcut_in_place=1 on the golden shortcut network: tensors that survive the pass equal the reference's, a tensor
+    written over holds its writer's output, and shortcuts of another shape than their connection keep their own tensor."""
+    from nebula_amd.net import Network
+    g = np.load(os.path.join(golden_dir, "resnet_shortcuts.npz"))
+    cfg = str(g["cfg"]).replace("[net]\n", "[net]\nfuse_shortcut=1\nshortcut_in_place=1\n", 1)
+    with Network(cfg) as net:
+        net.load_weight_blob(g["weights"])
+        net.set_input(g["input"])
+        net.forward()
+        kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
+        for i, k in enumerate(kinds):
+            w = net.output_writer(i)
+            if w == i:
+                assert rel(net.output(i), g["out_%02d" % i]) <= TOL, (i, k)
+            else:
+                assert w > i
+                if kinds[w] not in ("dropout_layer", "cost_layer"):
+                    assert rel(net.output(i), g["out_%02d" % w]) <= TOL, (i, k, w)
+
+
+def test_in_place_shortcut_is_refused_while_the_connection_is_still_read():
+    """Two shortcuts add the same tensor.  The first must not write over it (the second still reads it); the second may."""
+    from nebula_amd.net import Network
+    print("CASE in-place liveness", flush=True)
+    body = ("\n[convolutional]\nfilters=16\nsize=3\nstride=1\npadding=1\nactivation=relu\n"          # 0: the shared connection
+            "\n[convolutional]\nfilters=16\nsize=1\nstride=1\npadding=0\nactivation=relu\n"          # 1
+            "\n[convolutional]\nfilters=16\nsize=3\nstride=1\npadding=1\nactivation=linear\n"        # 2 (fused with 3)
+            "\n[shortcut]\nhops=3\nactivation=relu\n"                                                 # 3: adds layer 0
+            "\n[convolutional]\nfilters=16\nsize=3\nstride=1\npadding=1\nactivation=linear\n"        # 4 (fused with 5)
+            "\n[shortcut]\nhops=5\nactivation=relu\n"                                                 # 5: adds layer 0 again
+            "\n[avgpool]\nsize=12\nstride=12\npadding=0\n\n[connected]\noutput=10\nactivation=linear\n\n[softmax]\ngroups=1\n")
+    head = "[net]\nbatch=3\nheight=12\nwidth=12\nchannels=4\nconv_split=0\n%s"
+    rng = np.random.default_rng(23)
+    onet = ob.OracleNet(head % "" + body)
+    blob = _random_weights(onet.specs, rng)
+    x = rng.standard_normal((3, 4, 12, 12)).astype(np.float32)
+    onet.load_weights(blob)
+    ob.use_custom_gemm()
+    want = onet.forward(x)
+    with Network(head % "fuse_shortcut=1\nshortcut_in_place=1\n" + body) as net:
+        net.load_weight_blob(blob)
+        net.set_input(x)
+        net.forward()
+        assert net.output_writer(3) == 3          # kept its own tensor: layer 5 still needs layer 0
+        assert net.output_writer(0) == 5          # the last reader wrote over it
+        for i in (1, 3, 5, 6, 7, 8):
+            assert rel(net.output(i), want[i].ravel()) <= TOL, i
+        np.testing.assert_array_equal(net.output(0).view(np.uint32), net.output(5).view(np.uint32))

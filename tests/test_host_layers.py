@@ -107,3 +107,38 @@ def test_weights_round_trip_without_device(tmp_path):
         out = str(tmp_path / "out.wgh")
         assert netmod.lib().nbl_net_store_weights(net.h, out.encode()) == 0
         np.testing.assert_array_equal(np.fromfile(out, np.float32), g["weights"])
+
+
+def test_tensor_ownership_of_fused_and_in_place_shortcuts():
+    """Which layer's values a layer's output holds after a pass, decided at build time (no device needed): a fused
+    convolution shares its shortcut's tensor; with shortcut_in_place=1 a same-shape shortcut writes over its connection's
+    tensor unless a later layer still reads that tensor; a fusion is skipped while the convolution's own output is read."""
+    from nebula_amd.net import Network
+    from nebula_amd import zoo
+    conv = "\n[convolutional]\nfilters=16\nsize=3\nstride=1\npadding=1\nactivation=%s\n"
+    body = (conv % "relu" + conv % "relu" + conv % "linear" + "\n[shortcut]\nhops=3\nactivation=relu\n"      # 3 adds layer 0
+            + conv % "linear" + "\n[shortcut]\nhops=5\nactivation=relu\n"                                   # 5 adds layer 0 again
+            + "\n[avgpool]\nsize=12\nstride=12\npadding=0\n\n[connected]\noutput=10\nactivation=linear\n\n[softmax]\ngroups=1\n")
+    head = "[net]\nbatch=3\nheight=12\nwidth=12\nchannels=4\n%s"
+    writers = lambda cfg: [(lambda n: [n.output_writer(i) for i in range(n.num_layers)])(Network(cfg, device=-1))][0]
+    assert writers(head % "" + body) == list(range(9))
+    assert writers(head % "fuse_shortcut=1\n" + body) == [0, 1, 3, 3, 5, 5, 6, 7, 8]
+    # shortcut 3 keeps its tensor (layer 5 still reads layer 0), shortcut 5 takes layer 0's
+    assert writers(head % "fuse_shortcut=1\nshortcut_in_place=1\n" + body) == [5, 1, 3, 3, 5, 5, 6, 7, 8]
+    # in place needs the fusion
+    assert writers(head % "shortcut_in_place=1\n" + body) == list(range(9))
+    # shortcut 4 (hops=3) adds the output of convolution 1, so the pair (1, 2) cannot be fused: the sum would replace what
+    # shortcut 4 needs.  Shortcut 4 itself is fused with convolution 3 and may write over layer 1's tensor: its only other
+    # reader, shortcut 2, runs earlier.
+    twice = (conv % "relu" + conv % "linear" + "\n[shortcut]\nhops=2\nactivation=relu\n" + conv % "linear"
+             + "\n[shortcut]\nhops=3\nactivation=linear\n\n[softmax]\ngroups=1\n")
+    w = writers(head % "fuse_shortcut=1\nshortcut_in_place=1\n" + twice)
+    assert w == [0, 4, 2, 4, 4, 5], w
+    assert writers(head % "fuse_shortcut=1\n" + twice) == [0, 1, 2, 4, 4, 5]
+    # ResNet-50: sixteen fused convolutions; in place, every stage shares one tensor from its first block's output on
+    kinds = lambda n: [n.layer_info(i)["kind"] for i in range(n.num_layers)]
+    net = Network(zoo.resnet50_cfg(2, fuse_shortcut=True), device=-1)
+    assert sum(net.output_writer(i) != i for i in range(net.num_layers)) == 16
+    net = Network(zoo.resnet50_cfg(2, fuse_shortcut=True, in_place=True), device=-1)
+    sc = [i for i, k in enumerate(kinds(net)) if k == "shortcut_layer"]
+    assert [net.output_writer(i) for i in sc] == [13, 13, 13, 29, 29, 29, 29, 53, 53, 53, 53, 53, 53, 65, 65, 65]
