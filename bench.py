@@ -165,6 +165,50 @@ def single_conv(args):
     ctx.close()
 
 
+def conv_work_grid(args):
+    """The 64x64 tile of conv_igemm_kernel against how a launch is cut: output tiles per resident-block slot (6 slots per
+    CU) and k-tiles per tile.  256 filters on 16x16 maps (16 tiles per image, so the batch sets the tile count); a 3x3 layer
+    (tap-major gather) and a 1x1 layer (vector gather) at three depths each; tile shape pinned, no k-split."""
+    from nebula_amd import hip
+    ctx = hip.Ctx(0)
+    rng = np.random.default_rng(0)
+    F, HW, slots = 256, 16, 6 * 256
+    batches = [48, 96, 98, 192, 196, 384, 768]
+    rows = []
+    for k, pad, chans in ((3, 1, (16, 64, 128)), (1, 0, (128, 256, 512))):
+        for C_ in chans:
+            w = (rng.standard_normal((F, C_, k, k)) * np.sqrt(2.0 / (C_ * k * k))).astype(np.float32)
+            plan = ctx.conv_pack(w, np.zeros(F, np.float32), None, H=HW, W=HW, stride=1, pad=pad, act="relu")
+            plan.set_variant(4)
+            plan.set_split(0)
+            rec = {"layer": "%dx%d, %d channels" % (k, k, C_), "k_tiles_per_tile": C_ * k * k // 16, "tflops": {}}
+            for B in batches:
+                x = ctx.array(np.tile(rng.standard_normal((8, C_, HW, HW)).astype(np.float32), (B // 8 + 1, 1, 1, 1))[:B])
+                y = ctx.empty((B, F, HW, HW))
+                # the device takes some 50 ms of work to reach its sustained clock after an idle moment (the upload above)
+                ctx.timer_start()
+                for _ in range(3):
+                    plan(x, out=y)
+                est = max(ctx.timer_stop() / 3, 1e-3)
+                for _ in range(int(60.0 / est) + 1):
+                    plan(x, out=y)
+                ctx.sync()
+                reps = int(40.0 / est) + 1
+                ctx.timer_start()
+                for _ in range(reps):
+                    plan(x, out=y)
+                ms = ctx.timer_stop() / reps
+                assert plan.last_launch() == (4, 1)
+                rec["tflops"]["%.2f" % (16.0 * B / slots)] = round(plan.flop_per_image * B / ms / 1e9, 1)
+                x.free(); y.free()
+            log(rec)
+            rows.append(rec)
+    ctx.close()
+    print(json.dumps({"metric": "conv_igemm_kernel 64x64 tile, TFLOP/s by tiles per resident-block slot and k-tiles per tile",
+                      "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "tiles_per_slot": ["%.2f" % (16.0 * B / slots) for B in batches],
+                      "rows": rows}), flush=True)
+
+
 def image_input(args):
     """Device-side image preprocessing (nbl_image_to_input): 64 byte images of 375x500x3 -> 3x224x224 float planes."""
     from nebula_amd import hip
@@ -362,7 +406,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "images", "ptb", "memops"],
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "convgrid", "images", "ptb", "memops"],
                     help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
                          "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
                          "for counter passes over a single kernel")
@@ -388,6 +432,8 @@ def main():
         return copy_calibration(args)
     if args.workload == "conv":
         return single_conv(args)
+    if args.workload == "convgrid":
+        return conv_work_grid(args)
     if args.workload == "images":
         return image_input(args)
     if args.workload == "ptb":
