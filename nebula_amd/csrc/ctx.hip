@@ -188,6 +188,15 @@ __global__ void nbl_copy_kernel(uint4 *__restrict__ dst4, const uint4 *__restric
     if(i < ntail) dtail[i] = stail[i];
 }
 
+// The same copy with streaming stores (see nbl_stream_stores).
+__global__ void nbl_copy_stream_kernel(uint4 *__restrict__ dst4, const uint4 *__restrict__ src4, size_t n4,
+                                       unsigned char *__restrict__ dtail, const unsigned char *__restrict__ stail, unsigned ntail) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for(size_t j = i; j < n4; j += step) nbl_put<true>(dst4 + j, src4[j]);
+    if(i < ntail) dtail[i] = stail[i];
+}
+
 int nbl_copy_d2d(nbl_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
     if(!ctx) return NBL_EINVAL;
     if(bytes == 0) return NBL_OK;
@@ -199,9 +208,14 @@ int nbl_copy_d2d(nbl_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes)
     const unsigned ntail = (unsigned)(bytes % 16);
     size_t blocks = nbl_div_up_sz(n4 ? n4 : 1, 256);
     if(blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(nbl_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
-                       (uint4*)dst_dev, (const uint4*)src_dev, n4,
-                       (unsigned char*)dst_dev + n4 * 16, (const unsigned char*)src_dev + n4 * 16, ntail);
+    if(nbl_stream_stores(bytes, dst_dev, src_dev))
+        hipLaunchKernelGGL(nbl_copy_stream_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                           (uint4*)dst_dev, (const uint4*)src_dev, n4,
+                           (unsigned char*)dst_dev + n4 * 16, (const unsigned char*)src_dev + n4 * 16, ntail);
+    else
+        hipLaunchKernelGGL(nbl_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                           (uint4*)dst_dev, (const uint4*)src_dev, n4,
+                           (unsigned char*)dst_dev + n4 * 16, (const unsigned char*)src_dev + n4 * 16, ntail);
     NBL_LAUNCH_CHECK(ctx, "copy_d2d");
     return NBL_OK;
 }

@@ -79,7 +79,7 @@ void pool_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *_
 // fetched with ONE load of KS dwords at 4-byte alignment instead of KS loads (the address unit works per instruction,
 // and the general kernel's nine 4-byte loads per output held it to 40 % of the memory rate on these maps).
 template<int KS> struct __attribute__((packed, aligned(4))) WindowRow { float v[KS]; };
-template<bool IS_MAX, bool WRITE_INDEX, int KS>
+template<bool IS_MAX, bool WRITE_INDEX, int KS, bool STREAM>
 __global__ __launch_bounds__(256)
 void pool_inside_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
                         unsigned total, int H, int W, int OH, int OW, int stride) {
@@ -103,17 +103,18 @@ void pool_inside_kernel(const float *__restrict__ x, float *__restrict__ y, unsi
             }
         }
     if(IS_MAX) {
-        y[o] = best;
-        if(WRITE_INDEX) index[o] = best_at;
+        nbl_put<STREAM>(y + o, best);
+        if(WRITE_INDEX) nbl_put<STREAM>(index + o, best_at);
     } else {
-        y[o] = acc / (float)(KS * KS);
+        nbl_put<STREAM>(y + o, acc / (float)(KS * KS));
     }
 }
 
 // Stride 2, no padding, image width a multiple of 4: a lane produces two adjacent outputs from one
 // 16-byte load per window row (plus one scalar for the fifth column of a 3-wide window), so the
 // lanes of a wave read whole rows contiguously.  Same scan order, sentinel and tie rule as above.
-template<bool IS_MAX, bool WRITE_INDEX, int KS>
+// STREAM_IN (2-wide windows only: rows are read once) fetches the rows with streaming loads.
+template<bool IS_MAX, bool WRITE_INDEX, int KS, bool STREAM, bool STREAM_IN>
 __global__ __launch_bounds__(256)
 void pool_pair_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index,
                       unsigned total_pairs, int H, int W, int OH, int OW2) {
@@ -128,7 +129,7 @@ void pool_pair_kernel(const float *__restrict__ x, float *__restrict__ y, unsign
         const int ih = h0 + i;
         const bool row_ok = ih < H;
         const unsigned roff = base + (unsigned)((row_ok ? ih : 0) * W + w0);
-        const float4 q = *reinterpret_cast<const float4*>(x + roff);
+        const float4 q = nbl_get<STREAM_IN>(reinterpret_cast<const float4*>(x + roff));
         const float pad_v = IS_MAX ? -1e8f : 0.0f;
         v[i][0] = row_ok ? q.x : pad_v; v[i][1] = row_ok ? q.y : pad_v;
         v[i][2] = row_ok ? q.z : pad_v; v[i][3] = row_ok ? q.w : pad_v;
@@ -158,8 +159,8 @@ void pool_pair_kernel(const float *__restrict__ x, float *__restrict__ y, unsign
         at[p] = best_at;
     }
     const size_t o = (size_t)o2 * 2;
-    *reinterpret_cast<float2*>(y + o) = make_float2(out[0], out[1]);
-    if(IS_MAX && WRITE_INDEX) *reinterpret_cast<uint2*>(index + o) = make_uint2(at[0], at[1]);
+    nbl_put<STREAM>(reinterpret_cast<float2*>(y + o), out[0], out[1]);
+    if(IS_MAX && WRITE_INDEX) nbl_put<STREAM>(reinterpret_cast<uint2*>(index + o), at[0], at[1]);
 }
 
 // Average over whole planes (window = plane, stride = window, no padding: the pool that ends ResNet).  The
@@ -201,6 +202,7 @@ void avgpool_plane_kernel(const float *__restrict__ x, float *__restrict__ y, un
 // y = act(prev + conn') where conn' is conn cropped to the common channel/height/width box and
 // sampled with stride = max(1, in_w/out_w), sample = max(1, out_w/in_w) (common/utils.cc:28-60).
 // Fast path: identical spatial size (stride = sample = 1, same H and W), 4 elements per lane.
+template<bool STREAM, bool STREAM_IN>
 __global__ void shortcut_same_hw_kernel(const float4 *__restrict__ prev, const float4 *__restrict__ conn,
                                         float4 *__restrict__ y, size_t total4, unsigned hw4,
                                         unsigned in_c, unsigned out_c, int act) {
@@ -208,20 +210,20 @@ __global__ void shortcut_same_hw_kernel(const float4 *__restrict__ prev, const f
     if(e >= total4) return;
     const size_t plane = e / hw4;                  // b*out_c + c
     const unsigned c = (unsigned)(plane % out_c);
-    float4 v = prev[e];
+    float4 v = nbl_get<STREAM_IN>(prev + e);
     if(c < in_c) {
         const size_t b = plane / out_c;
-        const float4 r = conn[(b * in_c + c) * hw4 + (e - plane * hw4)];
+        const float4 r = nbl_get<STREAM_IN>(conn + (b * in_c + c) * hw4 + (e - plane * hw4));
         v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
     }
     v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
     v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
-    y[e] = v;
+    nbl_put<STREAM>(y + e, v);
 }
 
 // Spatial sizes differ by an integer stride and the output is not up-sampled (sample = 1): four
 // adjacent outputs per lane; with stride 2 their residuals are the even elements of 32 contiguous bytes.
-template<bool STRIDE2>
+template<bool STRIDE2, bool STREAM>
 __global__ void shortcut_strided_kernel(const float4 *__restrict__ prev, const float *__restrict__ conn,
                                         float4 *__restrict__ y, size_t total4,
                                         unsigned in_c, unsigned in_h, unsigned in_w,
@@ -246,7 +248,7 @@ __global__ void shortcut_strided_kernel(const float4 *__restrict__ prev, const f
     }
     v.x = nbl_act_apply(act, v.x); v.y = nbl_act_apply(act, v.y);
     v.z = nbl_act_apply(act, v.z); v.w = nbl_act_apply(act, v.w);
-    y[e] = v;
+    nbl_put<STREAM>(y + e, v);
 }
 
 __global__ void shortcut_general_kernel(const float *__restrict__ prev, const float *__restrict__ conn,
@@ -289,7 +291,7 @@ __device__ __forceinline__ float softmax_exp(float d) { return expf(d); }
 // Rows whose length is a multiple of 4 and whose start is 16-byte aligned, up to 1024 * PER4 entries: a thread keeps
 // PER4 pieces of four adjacent entries in registers (pieces tid, tid + 256, ...), so the row moves as 16-byte loads
 // and stores, once each way.
-template<int PER4>
+template<int PER4, bool STREAM>
 __global__ __launch_bounds__(256) void softmax_row_vec4_kernel(const float *__restrict__ x, float *__restrict__ y, unsigned n) {
     typedef float vec4 __attribute__((ext_vector_type(4)));
     __shared__ float red[4];
@@ -325,7 +327,10 @@ __global__ __launch_bounds__(256) void softmax_row_vec4_kernel(const float *__re
     #pragma unroll
     for(int i = 0; i < PER4; i++) {
         const unsigned j = tid + i * 256;
-        if(j < n4) out[j] = vec4{v[i][0] / s, v[i][1] / s, v[i][2] / s, v[i][3] / s};
+        if(j < n4) {
+            const vec4 q = vec4{v[i][0] / s, v[i][1] / s, v[i][2] / s, v[i][3] / s};
+            if constexpr(STREAM) __builtin_nontemporal_store(q, out + j); else out[j] = q;
+        }
     }
 }
 
@@ -592,20 +597,26 @@ int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index
     if(total == 0) return NBL_OK;
     if(total >= (1ull << 31) || in_total >= (1ull << 31))
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_pool_fwd: tensors of 2^31 elements or more are not supported");
+    const bool stream_out = nbl_stream_stores(total * sizeof(float), y_dev, x_dev);
     // two outputs per lane from 16-byte loads
     if(stride == 2 && pad == 0 && (ksize == 2 || ksize == 3) && W % 4 == 0 && OW == W / 2 && OW % 2 == 0 &&
        (((size_t)x_dev | (size_t)y_dev | (size_t)index_dev) & 15) == 0) {
         const unsigned pairs = (unsigned)(total / 2);
         dim3 pgrid(nbl_div_up(pairs, 256)), pblock(256);
+#define NBL_PAIR_LAUNCH_AS(IS_MAX, WI, KS, ST, SI) \
+        hipLaunchKernelGGL((pool_pair_kernel<IS_MAX, WI, KS, ST, SI>), pgrid, pblock, 0, ctx->stream, x_dev, y_dev, \
+                           index_dev, pairs, (int)H, (int)W, (int)OH, (int)(OW / 2))
 #define NBL_PAIR_LAUNCH(IS_MAX, WI, KS) \
-        hipLaunchKernelGGL((pool_pair_kernel<IS_MAX, WI, KS>), pgrid, pblock, 0, ctx->stream, x_dev, y_dev, index_dev, \
-                           pairs, (int)H, (int)W, (int)OH, (int)(OW / 2))
+        do { if(stream_out && KS == 2 && nbl_stream_loads(in_total * sizeof(float))) NBL_PAIR_LAUNCH_AS(IS_MAX, WI, KS, true, KS == 2); \
+             else if(stream_out) NBL_PAIR_LAUNCH_AS(IS_MAX, WI, KS, true, false); \
+             else NBL_PAIR_LAUNCH_AS(IS_MAX, WI, KS, false, false); } while(0)
         if(mode == NBL_POOL_MAX) {
             if(index_dev) { if(ksize == 2) NBL_PAIR_LAUNCH(true, true, 2); else NBL_PAIR_LAUNCH(true, true, 3); }
             else          { if(ksize == 2) NBL_PAIR_LAUNCH(true, false, 2); else NBL_PAIR_LAUNCH(true, false, 3); }
         } else {
             if(ksize == 2) NBL_PAIR_LAUNCH(false, false, 2); else NBL_PAIR_LAUNCH(false, false, 3);
         }
+#undef NBL_PAIR_LAUNCH_AS
 #undef NBL_PAIR_LAUNCH
         NBL_LAUNCH_CHECK(ctx, "pool_pair_kernel");
         return NBL_OK;
@@ -623,8 +634,10 @@ int nbl_pool_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned *index
     // every tap of every window inside the image: one load per window row
     if(pad == 0 && (ksize == 2 || ksize == 3) && (OH - 1) * stride + ksize <= H && (OW - 1) * stride + ksize <= W) {
 #define NBL_INSIDE_LAUNCH(IS_MAX, WI, KS) \
-        hipLaunchKernelGGL((pool_inside_kernel<IS_MAX, WI, KS>), grid, block, 0, ctx->stream, x_dev, y_dev, index_dev, \
-                           (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)stride)
+        do { if(stream_out) hipLaunchKernelGGL((pool_inside_kernel<IS_MAX, WI, KS, true>), grid, block, 0, ctx->stream, x_dev, y_dev, \
+                                               index_dev, (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)stride); \
+             else hipLaunchKernelGGL((pool_inside_kernel<IS_MAX, WI, KS, false>), grid, block, 0, ctx->stream, x_dev, y_dev, \
+                                     index_dev, (unsigned)total, (int)H, (int)W, (int)OH, (int)OW, (int)stride); } while(0)
         if(mode == NBL_POOL_MAX) {
             if(index_dev) { if(ksize == 2) NBL_INSIDE_LAUNCH(true, true, 2); else NBL_INSIDE_LAUNCH(true, true, 3); }
             else          { if(ksize == 2) NBL_INSIDE_LAUNCH(true, false, 2); else NBL_INSIDE_LAUNCH(true, false, 3); }
@@ -663,6 +676,7 @@ int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev,
     const size_t total = (size_t)B * out_c * out_h * out_w;
     if(total >= (1ull << 40)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_shortcut_fwd: tensor too large");
     const unsigned hw = out_h * out_w;
+    const bool stream_out = nbl_stream_stores(total * sizeof(float), y_dev, prev_dev, conn_dev);
     const bool same_hw = in_h == out_h && in_w == out_w;
     bool vec = same_hw && hw % 4 == 0 && (((size_t)prev_dev | (size_t)conn_dev | (size_t)y_dev) & 15) == 0;
     unsigned hw4 = hw / 4, vin_c = in_c, vout_c = out_c;
@@ -679,20 +693,24 @@ int nbl_shortcut_fwd(nbl_ctx *ctx, const float *prev_dev, const float *conn_dev,
                              (stride != 2 || in_w % 4 == 0);
     if(vec) {
         const size_t total4 = total / 4;
-        hipLaunchKernelGGL(shortcut_same_hw_kernel, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0, ctx->stream,
-                           (const float4*)prev_dev, (const float4*)conn_dev, (float4*)y_dev, total4, hw4,
-                           vin_c, vout_c, act);
+        const size_t read_bytes = (total + (size_t)B * (in_c < out_c ? in_c : out_c) * hw) * sizeof(float);
+#define NBL_SAME_HW_LAUNCH(ST, SI) \
+        hipLaunchKernelGGL((shortcut_same_hw_kernel<ST, SI>), dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0, ctx->stream, \
+                           (const float4*)prev_dev, (const float4*)conn_dev, (float4*)y_dev, total4, hw4, vin_c, vout_c, act)
+        if(stream_out && nbl_stream_loads(read_bytes)) NBL_SAME_HW_LAUNCH(true, true);
+        else if(stream_out) NBL_SAME_HW_LAUNCH(true, false);
+        else NBL_SAME_HW_LAUNCH(false, false);
+#undef NBL_SAME_HW_LAUNCH
     } else if(strided_vec) {
         const size_t total4 = total / 4;
         const unsigned box_c = in_c < out_c ? in_c : out_c, box_h = in_h < out_h ? in_h : out_h;
-        if(stride == 2)
-            hipLaunchKernelGGL(shortcut_strided_kernel<true>, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0,
-                               ctx->stream, (const float4*)prev_dev, conn_dev, (float4*)y_dev, total4, in_c, in_h, in_w,
-                               out_c, out_h, out_w / 4, stride, box_c, box_h, act);
-        else
-            hipLaunchKernelGGL(shortcut_strided_kernel<false>, dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0,
-                               ctx->stream, (const float4*)prev_dev, conn_dev, (float4*)y_dev, total4, in_c, in_h, in_w,
-                               out_c, out_h, out_w / 4, stride, box_c, box_h, act);
+#define NBL_STRIDED_LAUNCH(S2, ST) \
+        hipLaunchKernelGGL((shortcut_strided_kernel<S2, ST>), dim3((unsigned)nbl_div_up_sz(total4, 256)), dim3(256), 0, \
+                           ctx->stream, (const float4*)prev_dev, conn_dev, (float4*)y_dev, total4, in_c, in_h, in_w, \
+                           out_c, out_h, out_w / 4, stride, box_c, box_h, act)
+        if(stride == 2) { if(stream_out) NBL_STRIDED_LAUNCH(true, true); else NBL_STRIDED_LAUNCH(true, false); }
+        else            { if(stream_out) NBL_STRIDED_LAUNCH(false, true); else NBL_STRIDED_LAUNCH(false, false); }
+#undef NBL_STRIDED_LAUNCH
     } else {
         hipLaunchKernelGGL(shortcut_general_kernel, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
                            prev_dev, conn_dev, y_dev, total, in_c, in_h, in_w, out_c, out_h, out_w, stride, sample,
@@ -708,7 +726,10 @@ int nbl_softmax_fwd(nbl_ctx *ctx, const float *x_dev, float *y_dev, unsigned row
     if(rows == 0 || n == 0) return NBL_OK;
     if(n % 4 == 0 && n <= 16384 && (((size_t)x_dev | (size_t)y_dev) & 15) == 0) {
         const unsigned per4 = nbl_div_up(n / 4, 256);
-#define NBL_SOFTMAX_VEC(P) hipLaunchKernelGGL((softmax_row_vec4_kernel<P>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n)
+        const bool stream_out = nbl_stream_stores((size_t)rows * n * sizeof(float), y_dev, x_dev);
+#define NBL_SOFTMAX_VEC(P) \
+        do { if(stream_out) hipLaunchKernelGGL((softmax_row_vec4_kernel<P, true>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n); \
+             else hipLaunchKernelGGL((softmax_row_vec4_kernel<P, false>), dim3(rows), dim3(256), 0, ctx->stream, x_dev, y_dev, n); } while(0)
         if(per4 <= 1) NBL_SOFTMAX_VEC(1); else if(per4 <= 2) NBL_SOFTMAX_VEC(2); else if(per4 <= 4) NBL_SOFTMAX_VEC(4);
         else if(per4 <= 6) NBL_SOFTMAX_VEC(6); else if(per4 <= 8) NBL_SOFTMAX_VEC(8); else if(per4 <= 10) NBL_SOFTMAX_VEC(10);
         else if(per4 <= 12) NBL_SOFTMAX_VEC(12); else NBL_SOFTMAX_VEC(16);

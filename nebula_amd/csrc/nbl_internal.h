@@ -43,6 +43,59 @@ static inline unsigned nbl_div_up(unsigned a, unsigned b) { return (a + b - 1) /
 static inline size_t nbl_div_up_sz(size_t a, size_t b) { return (a + b - 1) / b; }
 
 // -------------------------------------------------------------------------------------------------
+// Streaming stores.  A kernel that writes a tensor it does not read (out of place) keeps 69 % of the memory rate with
+// ordinary stores and 88 % with non-temporal ones on this part (256 MiB copy: 98 us against 76 us); a kernel that
+// writes the lines it has just read loses with them (76 us against 89 us), and so does a producer whose consumer
+// would have found the tensor in the caches.  Kernels take STREAM as a template argument and the launch site decides
+// with nbl_stream_stores(): the output must not alias an input and must be at least NBL_STREAM_MIN_BYTES long, the
+// capacity of the eight L2 caches together (a shorter tensor may still be there when the next kernel reads it; whole
+// networks time the same either way, so the line is drawn where the isolated kernel starts to gain).
+// -------------------------------------------------------------------------------------------------
+#ifndef NBL_STREAM_MIN_BYTES
+#define NBL_STREAM_MIN_BYTES ((size_t)32 << 20)
+#endif
+static inline bool nbl_stream_stores(size_t bytes_written, const void *out, const void *in0, const void *in1 = NULL) {
+    return bytes_written >= NBL_STREAM_MIN_BYTES && out != in0 && out != in1;
+}
+// Streaming loads pay only where nothing is read twice and the data cannot already sit in the 256 MiB memory-side cache:
+// the 2x2 pool of a 411 MB tensor gains 8 % and the same-shape shortcut of two 205 MB tensors 6 %, while a 3x3/2 pool
+// (adjacent windows share rows) loses 60 % and a 164 MB softmax 13 %.
+#ifndef NBL_STREAM_IN_MIN_BYTES
+#define NBL_STREAM_IN_MIN_BYTES ((size_t)256 << 20)
+#endif
+static inline bool nbl_stream_loads(size_t bytes_read) { return bytes_read >= NBL_STREAM_IN_MIN_BYTES; }
+typedef float    nbl_f32x4 __attribute__((ext_vector_type(4)));
+typedef float    nbl_f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned nbl_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned nbl_u32x2 __attribute__((ext_vector_type(2)));
+template<bool STREAM> __device__ __forceinline__ void nbl_put(float *p, float v) {
+    if constexpr(STREAM) __builtin_nontemporal_store(v, p); else *p = v;
+}
+template<bool STREAM> __device__ __forceinline__ void nbl_put(unsigned *p, unsigned v) {
+    if constexpr(STREAM) __builtin_nontemporal_store(v, p); else *p = v;
+}
+template<bool STREAM> __device__ __forceinline__ void nbl_put(float2 *p, float a, float b) {
+    if constexpr(STREAM) __builtin_nontemporal_store(nbl_f32x2{a, b}, reinterpret_cast<nbl_f32x2*>(p)); else *p = make_float2(a, b);
+}
+template<bool STREAM> __device__ __forceinline__ void nbl_put(uint2 *p, unsigned a, unsigned b) {
+    if constexpr(STREAM) __builtin_nontemporal_store(nbl_u32x2{a, b}, reinterpret_cast<nbl_u32x2*>(p)); else *p = make_uint2(a, b);
+}
+template<bool STREAM> __device__ __forceinline__ void nbl_put(float4 *p, float4 v) {
+    if constexpr(STREAM) __builtin_nontemporal_store(nbl_f32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<nbl_f32x4*>(p)); else *p = v;
+}
+template<bool STREAM> __device__ __forceinline__ float4 nbl_get(const float4 *p) {
+    if constexpr(STREAM) {
+        const nbl_f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nbl_f32x4*>(p));
+        return make_float4(t.x, t.y, t.z, t.w);
+    } else {
+        return *p;
+    }
+}
+template<bool STREAM> __device__ __forceinline__ void nbl_put(uint4 *p, uint4 v) {
+    if constexpr(STREAM) __builtin_nontemporal_store(nbl_u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<nbl_u32x4*>(p)); else *p = v;
+}
+
+// -------------------------------------------------------------------------------------------------
 // The thirteen activations of common/activations.cc:6-89, evaluated as the CPU file does: the
 // literals there are doubles, so anything that touches one is computed in double and rounded once
 // on the store.  relu / leaky / relie keep the `x > 0` predicate on the float value, which is what

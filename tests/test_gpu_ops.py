@@ -225,6 +225,12 @@ def test_copy_d2d(ctx):
         src, dst = ctx.array(a), ctx.array(np.zeros(n, np.float32))
         ctx.copy(dst, src)
         np.testing.assert_array_equal(bits(dst.numpy()), bits(a))
+    # a copy long enough for the streaming-store kernel (32 MiB and more), with a ragged tail
+    n = (40 << 20) // 4 + 3
+    a = rng.standard_normal(n).astype(np.float32)
+    src, dst = ctx.array(a), ctx.array(np.zeros(n, np.float32))
+    ctx.copy(dst, src)
+    np.testing.assert_array_equal(bits(dst.numpy()), bits(a))
     big = ctx.array(np.arange(64, dtype=np.float32))
     rc = hip.lib().nbl_copy_d2d(ctx.h, big.ptr + 16, big.ptr, 64)
     assert rc == -1 and b"overlap" in hip.lib().nbl_last_error(ctx.h)
@@ -245,7 +251,10 @@ POOL = [(2, 3, 12, 12, 3, 2, 1), (2, 2, 13, 11, 3, 2, 0), (1, 4, 8, 8, 2, 2, 0),
         # rows that are not whole 16-byte pieces (AlexNet's maps): odd plane counts, padding, stride 1, a 5x5 window, a
         # non-square plane, and AlexNet's first pool at its full size
         (5, 23, 27, 27, 3, 2, 0), (16, 40, 13, 13, 3, 2, 0), (4, 24, 27, 27, 3, 2, 1), (2, 12, 55, 55, 2, 1, 1),
-        (3, 24, 31, 31, 5, 3, 2), (4, 10, 45, 39, 3, 2, 0), (128, 96, 55, 55, 3, 2, 0)]
+        (3, 24, 31, 31, 5, 3, 2), (4, 10, 45, 39, 3, 2, 0), (128, 96, 55, 55, 3, 2, 0),
+        # outputs of 32 MiB and more leave through streaming stores: ResNet's pool at batch 64, a 2x2 pool of VGG-16's
+        # first; a 2x2 pool whose input is longer than 256 MiB also arrives through streaming loads
+        (64, 64, 112, 112, 3, 2, 0), (16, 64, 224, 224, 2, 2, 0), (22, 64, 224, 224, 2, 2, 0)]
 
 
 @pytest.mark.parametrize("geom", POOL)
@@ -309,7 +318,13 @@ def test_avgpool_whole_plane_bit_exact(ctx, geom):
 SHORTCUT = [((2, 4, 9, 9), (2, 16, 9, 9)), ((2, 8, 10, 10), (2, 16, 5, 5)), ((1, 6, 19, 19), (1, 6, 10, 10)),
             ((2, 8, 4, 4), (2, 4, 8, 8)), ((3, 5, 7, 7), (3, 5, 7, 7)), ((2, 16, 8, 8), (2, 16, 8, 8)),
             ((2, 8, 12, 12), (2, 32, 12, 12)), ((2, 32, 12, 12), (2, 8, 12, 12)), ((2, 8, 7, 7), (2, 8, 7, 7)),
-            ((2, 8, 16, 16), (2, 24, 8, 8)), ((2, 6, 24, 24), (2, 6, 8, 8)), ((2, 4, 12, 12), (2, 8, 4, 4))]
+            ((2, 8, 16, 16), (2, 24, 8, 8)), ((2, 6, 24, 24), (2, 6, 8, 8)), ((2, 4, 12, 12), (2, 8, 4, 4)),
+            # outputs of 32 MiB and more (streaming stores out of place, ordinary ones in place): same shape, more
+            # output channels than the connection has, a ResNet stage entry (stride 2), stride 3
+            ((64, 256, 28, 28), (64, 256, 28, 28)), ((32, 128, 28, 28), (32, 512, 28, 28)),
+            ((32, 256, 56, 56), (32, 512, 28, 28)), ((16, 64, 84, 84), (16, 768, 28, 28)),
+            # 2 x 205 MB read: streaming loads as well
+            ((64, 256, 56, 56), (64, 256, 56, 56))]
 
 
 @pytest.mark.parametrize("dims", SHORTCUT)
@@ -376,7 +391,8 @@ def test_bias_and_batchnorm_primitives(ctx):
 
 # row lengths either side of every kernel choice (4, 8 or 16 entries per thread in registers, then the general kernel)
 @pytest.mark.parametrize("shape", [(6, 333), (64, 1000), (3, 10000), (1, 5), (128, 1000), (2, 1024), (2, 1025), (3, 2048),
-                                   (2, 2049), (2, 8713), (2, 16384), (2, 16385), (3, 20000), (5, 1)])
+                                   (2, 2049), (2, 8713), (2, 16384), (2, 16385), (3, 20000), (5, 1),
+                                   (1024, 10000)])      # 39 MiB: leaves through streaming stores
 def test_softmax(ctx, shape):
     announce("softmax", shape)
     rng = np.random.default_rng(shape[1])
