@@ -442,21 +442,25 @@ void conv_igemm_kernel(const ConvArgs a) {
     // always applied (it is 1.0 where the layer has no batch normalisation, and acc * 1 + b rounds as
     // acc + b does).
     // (forced inline: called from four places, and as a real call it would take the accumulators through memory)
-    auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff, unsigned roff, int act, int post_act)
-                          __attribute__((always_inline)) {
+    typedef float __attribute__((ext_vector_type(NT))) pixvec;
+    // Tiles of up to 64 accumulator registers per lane request their residual rows before the last two k-tiles
+    // (prefetch_residual) and hand them to the epilogue in registers; larger tiles have no registers to spare for that
+    // (they spill) and load them in the epilogue, one group of rows ahead.
+    constexpr bool PREFETCH_RES = MT * NT <= 2;
+    constexpr int NPRE = PREFETCH_RES ? 16 * MT : 1;
+    auto short_epilogue = [&](auto sloped, auto with_residual, int f_lane, unsigned yoff, unsigned roff, unsigned res_pitch,
+                              const pixvec (&rpre)[NPRE], int act, int post_act) __attribute__((always_inline)) {
         // sloped: 0 relu / linear through selects on uniform flags, 1 leaky / relie as well, 2 the ReLU network's two
         //         cases resolved at compile time: relu without a residual, or linear + residual + relu (one max each)
-        // with_residual: 0 none, 1 at the output's own offsets (same shape), 2 at offsets of its own
+        // with_residual: 0 none, 1 rows res_pitch bytes apart from byte offset roff (in rpre already when PREFETCH_RES)
         constexpr bool SLOPED = decltype(sloped)::value == 1, RELU_NET = decltype(sloped)::value == 2,
-                       RES = decltype(with_residual)::value != 0, RES_OWN = decltype(with_residual)::value == 2;
-        typedef float __attribute__((ext_vector_type(NT))) pixvec;
+                       RES = decltype(with_residual)::value != 0;
         const unsigned row_bytes = (unsigned)a.OHW * 4u;
-        const unsigned res_row_bytes = (unsigned)a.res_hw * 4u;
+        const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(RES ? a.res : a.y), 0, (int)0xffffffffu, 0x00020000);
         // Output rows (and residual rows) go through buffer descriptors: the lane's own offset is a constant vector
         // offset, the row's offset is uniform and rides in the scalar offset -- no address arithmetic per row.  (Both
         // tensors are below 4 GiB here, which is what selects this epilogue.)
         const __amdgpu_buffer_rsrc_t yres = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, (int)0xffffffffu, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(RES ? a.res : a.y), 0, (int)0xffffffffu, 0x00020000);
         // per-filter constants one group of rows ahead of their use
         vec4f gv[2][MT], bv[2][MT];
         auto load_constants = [&](int q) {
@@ -474,9 +478,13 @@ void conv_igemm_kernel(const ConvArgs a) {
             if(RES) {
                 #pragma unroll
                 for(int e = 0; e < 4 * MT; e++) {
-                    const unsigned row = (unsigned)(q * 8 * MT + e) * (RES_OWN ? res_row_bytes : row_bytes);       // uniform
-                    if constexpr(NT == 1) rv[e][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rres, (int)(RES_OWN ? roff : yoff), (int)row, 0));
-                    else rv[e] = __builtin_bit_cast(pixvec, __builtin_amdgcn_raw_buffer_load_b64(rres, (int)(RES_OWN ? roff : yoff), (int)row, 0));
+                    if constexpr(PREFETCH_RES) {
+                        rv[e] = rpre[q * 4 * MT + e];
+                    } else {
+                        const unsigned row = (unsigned)(q * 8 * MT + e) * res_pitch;       // uniform
+                        if constexpr(NT == 1) rv[e][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rres, (int)roff, (int)row, 0));
+                        else rv[e] = __builtin_bit_cast(pixvec, __builtin_amdgcn_raw_buffer_load_b64(rres, (int)roff, (int)row, 0));
+                    }
                 }
             }
             #pragma unroll
@@ -503,63 +511,98 @@ void conv_igemm_kernel(const ConvArgs a) {
         }
     };
 
-    // Epilogue of one finished output tile: y = act(acc * g[f] + b[f]) (+ fused shortcut).
-    // Accumulator register r of a 32x32 MFMA tile holds tile row 8*(r/4) + 4*(lane/32) + r%4 and tile
-    // column lane%32; with the interleaving above that is filter row*MT + i and pixel (lane%32)*NT + j
-    // of the wave's sub-tile.
-    auto epilogue = [&](int tile) {
+    // Where a finished tile goes, decided before the last two k-tiles are multiplied so that the residual rows of a
+    // fused shortcut can be requested then and arrive under that work instead of after it.
+    // Short epilogue: every filter row of the tile exists, the lane's NT pixels are one aligned
+    // vector (OH*OW even keeps pairs inside one image), and rows are reached as base pointer +
+    // 32-bit offset, so a row costs one integer add besides its arithmetic.  An instruction spent
+    // here is an instruction the matrix pipe waits for, which is what layers with few patch rows
+    // are made of.
+    // A fused shortcut with fewer channels than filters gives a tile's rows a residual either all or not at
+    // all (mixed tiles take the general path); a tile without one applies the two activations in a row, which
+    // is one activation when either is linear.  A strided or larger connection is read at its own row pitch;
+    // pairs of pixels (NT = 2) are one vector of it only at stride 1 and equal width.
+    struct EpiloguePlan {
+        bool lane_live, use_short, tile_res;
+        int f_lane, act, post_act;
+        unsigned yoff, roff, res_pitch;       // byte offsets of the lane's first row; bytes between residual rows
+    };
+    auto plan_epilogue = [&]() {
+        EpiloguePlan p;
         const int m0 = tile_m * BM, n0 = tile_n * BN;
         const int nbase = n0 + wn * NT * 32 + l32 * NT;
-        if(nbase >= a.N) return;
-        const int b0 = (int)a.div_ohw.div((unsigned)nbase), pix0 = nbase - b0 * a.OHW;
-        // Short epilogue: every filter row of the tile exists, the lane's NT pixels are one aligned
-        // vector (OH*OW even keeps pairs inside one image), and rows are reached as base pointer +
-        // 32-bit offset, so a row costs one integer add besides its arithmetic.  An instruction spent
-        // here is an instruction the matrix pipe waits for, which is what layers with few patch rows
-        // are made of.
-        // A fused shortcut with fewer channels than filters gives a tile's rows a residual either all or not at
-        // all (mixed tiles take the general path); a tile without one applies the two activations in a row, which
-        // is one activation when either is linear.  A strided or larger connection is read at its own row pitch;
-        // pairs of pixels (NT = 2) are one vector of it only at stride 1 and equal width.
-        const bool tile_res = a.res != NULL && m0 + BM <= a.res_c, tile_plain = a.res == NULL || m0 >= a.res_c;
-        if(a.short_epilogue && m0 + BM <= a.F && (NT == 1 || (a.OHW & 1) == 0) && (tile_res || tile_plain) &&
-           (!tile_res || NT == 1 || (a.res_stride == 1 && a.res_hw == a.OHW)) &&
-           (!tile_plain || a.res == NULL || a.act == NBL_ACT_LINEAR || a.post_act == NBL_ACT_LINEAR)) {
-            const int f_lane = m0 + wm * MT * 32 + half * 4 * MT;
-            const unsigned yoff = ((unsigned)(b0 * a.F + f_lane) * (unsigned)a.OHW + (unsigned)pix0) * 4u;
-            unsigned roff = 0;
-            int act = a.act, post_act = a.post_act;
-            if(tile_res) {
+        p.lane_live = nbase < a.N;
+        const int nb = p.lane_live ? nbase : 0;
+        const int b0 = (int)a.div_ohw.div((unsigned)nb), pix0 = nb - b0 * a.OHW;
+        p.tile_res = a.res != NULL && m0 + BM <= a.res_c;
+        const bool tile_plain = a.res == NULL || m0 >= a.res_c;
+        p.use_short = FAST_ACT && a.short_epilogue && m0 + BM <= a.F && (NT == 1 || (a.OHW & 1) == 0) && (p.tile_res || tile_plain) &&
+                      (!p.tile_res || NT == 1 || (a.res_stride == 1 && a.res_hw == a.OHW)) &&
+                      (!tile_plain || a.res == NULL || a.act == NBL_ACT_LINEAR || a.post_act == NBL_ACT_LINEAR);
+        p.f_lane = m0 + wm * MT * 32 + half * 4 * MT;
+        p.yoff = ((unsigned)(b0 * a.F + p.f_lane) * (unsigned)a.OHW + (unsigned)pix0) * 4u;
+        p.roff = p.yoff;
+        p.res_pitch = (unsigned)a.OHW * 4u;
+        p.act = a.act; p.post_act = a.post_act;
+        if(p.tile_res) {
+            const bool res_same_shape = a.res_c == a.F && a.res_hw == a.OHW && a.res_stride == 1;   // uniform
+            if(!res_same_shape) {
                 unsigned rpix = (unsigned)pix0;
                 if(a.res_hw != a.OHW || a.res_stride != 1) {
                     const int h = (int)a.div_ow.div((unsigned)pix0), w = pix0 - h * a.OW;
                     rpix = (unsigned)(h * a.res_stride * a.res_w + w * a.res_stride);
                 }
-                roff = ((unsigned)(b0 * a.res_c + f_lane) * (unsigned)a.res_hw + rpix) * 4u;
-            } else if(a.res != NULL) {
-                act = a.act == NBL_ACT_LINEAR ? a.post_act : a.act;
-                post_act = NBL_ACT_LINEAR;
+                p.roff = ((unsigned)(b0 * a.res_c + p.f_lane) * (unsigned)a.res_hw + rpix) * 4u;
+                p.res_pitch = (unsigned)a.res_hw * 4u;
             }
+        } else if(a.res != NULL) {
+            p.act = a.act == NBL_ACT_LINEAR ? a.post_act : a.act;
+            p.post_act = NBL_ACT_LINEAR;
+        }
+        return p;
+    };
+    // The 16 * MT residual rows of this lane (row q * 8 * MT + e of the lane's filters sits in entry q * 4 * MT + e).
+    // A block reads only the residual of the tile it writes itself, so an output written over the connection is safe.
+    auto prefetch_residual = [&](const EpiloguePlan &p, pixvec (&rpre)[NPRE]) {
+        if(!PREFETCH_RES || !(p.lane_live && p.use_short && p.tile_res)) return;
+        const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.res), 0, (int)0xffffffffu, 0x00020000);
+        #pragma unroll
+        for(int q = 0; q < 4; q++) {
+            #pragma unroll
+            for(int e = 0; e < 4 * MT; e++) {
+                const unsigned row = (unsigned)(q * 8 * MT + e) * p.res_pitch;       // uniform
+                constexpr int at = PREFETCH_RES ? 4 * MT : 0;       // (keeps the index inside the one-entry array of the other case)
+                if constexpr(NT == 1) rpre[q * at + (PREFETCH_RES ? e : 0)][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rres, (int)p.roff, (int)row, 0));
+                else rpre[q * at + (PREFETCH_RES ? e : 0)] = __builtin_bit_cast(pixvec, __builtin_amdgcn_raw_buffer_load_b64(rres, (int)p.roff, (int)row, 0));
+            }
+        }
+    };
+
+    // Epilogue of one finished output tile: y = act(acc * g[f] + b[f]) (+ fused shortcut).
+    // Accumulator register r of a 32x32 MFMA tile holds tile row 8*(r/4) + 4*(lane/32) + r%4 and tile
+    // column lane%32; with the interleaving above that is filter row*MT + i and pixel (lane%32)*NT + j
+    // of the wave's sub-tile.
+    auto epilogue = [&](const EpiloguePlan &p, const pixvec (&rpre)[NPRE]) {
+        if(!p.lane_live) return;
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+        const int nbase = n0 + wn * NT * 32 + l32 * NT;
+        const int b0 = (int)a.div_ohw.div((unsigned)nbase), pix0 = nbase - b0 * a.OHW;
+        if constexpr(FAST_ACT) if(p.use_short) {       // (the host selects the short epilogue for the cheap activations only)
             typedef std::integral_constant<int, 0> no_res;
-            typedef std::integral_constant<int, 1> res_at_output;
-            typedef std::integral_constant<int, 2> res_own;
-            const bool res_same_shape = a.res_c == a.F && a.res_hw == a.OHW && a.res_stride == 1;   // uniform
+            typedef std::integral_constant<int, 1> with_res;
             typedef std::integral_constant<int, 0> flags; typedef std::integral_constant<int, 1> slopes; typedef std::integral_constant<int, 2> relu_net;
             // (uniform) the two forms a ReLU network's layers take: relu alone, or linear + residual + relu
-            const bool is_relu_net = a.short_epilogue == 1 && (tile_res ? act == NBL_ACT_LINEAR && post_act == NBL_ACT_RELU
-                                                                        : act == NBL_ACT_RELU && post_act == NBL_ACT_LINEAR);
+            const bool is_relu_net = a.short_epilogue == 1 && (p.tile_res ? p.act == NBL_ACT_LINEAR && p.post_act == NBL_ACT_RELU
+                                                                          : p.act == NBL_ACT_RELU && p.post_act == NBL_ACT_LINEAR);
             if(is_relu_net) {
-                if(!tile_res) short_epilogue(relu_net(), no_res(), f_lane, yoff, roff, act, post_act);
-                else if(res_same_shape) short_epilogue(relu_net(), res_at_output(), f_lane, yoff, roff, act, post_act);
-                else short_epilogue(relu_net(), res_own(), f_lane, yoff, roff, act, post_act);
+                if(!p.tile_res) short_epilogue(relu_net(), no_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
+                else short_epilogue(relu_net(), with_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
             } else if(a.short_epilogue == 1) {
-                if(!tile_res) short_epilogue(flags(), no_res(), f_lane, yoff, roff, act, post_act);
-                else if(res_same_shape) short_epilogue(flags(), res_at_output(), f_lane, yoff, roff, act, post_act);
-                else short_epilogue(flags(), res_own(), f_lane, yoff, roff, act, post_act);
+                if(!p.tile_res) short_epilogue(flags(), no_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
+                else short_epilogue(flags(), with_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
             } else {
-                if(!tile_res) short_epilogue(slopes(), no_res(), f_lane, yoff, roff, act, post_act);
-                else if(res_same_shape) short_epilogue(slopes(), res_at_output(), f_lane, yoff, roff, act, post_act);
-                else short_epilogue(slopes(), res_own(), f_lane, yoff, roff, act, post_act);
+                if(!p.tile_res) short_epilogue(slopes(), no_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
+                else short_epilogue(slopes(), with_res(), p.f_lane, p.yoff, p.roff, p.res_pitch, rpre, p.act, p.post_act);
             }
             return;
         }
@@ -731,11 +774,17 @@ void conv_igemm_kernel(const ConvArgs a) {
         ld_next(st1);
         tile_step(st0, 0);
     }
-    // last pair: nothing left to load
+    // last pair: nothing left to load but the residual rows the epilogue will add
+    pixvec rpre[NPRE];
+    EpiloguePlan plan;
+    if(!split_block) {
+        plan = plan_epilogue();
+        prefetch_residual(plan, rpre);
+    }
     tile_step(st1, 1);
     mfma_steps(cur, ks_first(), ks_last());
     if(split_block) store_partial();
-    else epilogue(tile);
+    else epilogue(plan, rpre);
 }
 
 // Second half of a k-split convolution: adds the parts in order and applies the epilogue the whole-tile
