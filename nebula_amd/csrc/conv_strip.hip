@@ -34,7 +34,7 @@ constexpr size_t STRIP_LDS_LIMIT = 80 * 1024;     // two blocks per CU (160 KB o
 struct StripArgs {
     const float *x; const float *wq; const float *g; const float *b; float *y; const int *otab;
     int C, H, W, F, OW, OHW, stride, pad;
-    int Kp, Mp, tiles_m, tiles_per_image;
+    int K, Kp, Mp, tiles_m, tiles_per_image;
     int rows, pitch;
     int act;
     int runs;               // pixel tiles of the launch (tiles_per_image * batch)
@@ -120,7 +120,7 @@ void conv_strip_kernel(const StripArgs a) {
     const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.wq), 0, (int)((unsigned)a.Kp * (unsigned)a.Mp * 4u), 0x00020000);
     const unsigned w_lane = (unsigned)(half * a.Mp + m0 + l32 * MT) * 16u;
     const unsigned w_step = (unsigned)a.Mp * 32u;           // two quads of k per step
-    const int nsteps = a.Kp / 8;
+    const int nsteps = (a.K + 7) / 8;     // steps of 8 patch rows; the packed weights are zero from row K to row Kp
     auto load_a = [&](vec4f (&dst)[MT], int s) {
         #pragma unroll
         for(int i = 0; i < MT; i++)
@@ -141,7 +141,7 @@ void conv_strip_kernel(const StripArgs a) {
     // Software pipeline, written out over four steps so that every stage lives in registers of its own and nothing
     // is moved: the weights of step s+3 and the strip offsets of step s+2 are requested at the start of step s, the
     // strip values of step s+1 are read (with the offsets requested a step earlier) before the MFMAs of step s issue.
-    // Kp is a multiple of 32, so the number of steps is a multiple of 4; requests past the end repeat the last step.
+    // Requests past the end repeat the last step; the steps of the last round past the end are skipped (uniform test).
     vec4f wa[4][MT];
     vec4i off[4];
     float bv[2][4];
@@ -153,7 +153,7 @@ void conv_strip_kernel(const StripArgs a) {
     off[1] = tab4[2 * min(1, last)];
     load_b(bv[0], off[0]);
 #define NBL_STRIP_STEP(U)                                                                                   \
-    {                                                                                                       \
+    if(U == 0 || s + U < nsteps) {                                                                          \
         load_a(wa[(U + 3) & 3], min(s + U + 3, last));                                                      \
         off[(U + 2) & 3] = tab4[2 * min(s + U + 2, last)];                                                  \
         load_b(bv[(U + 1) & 1], off[(U + 1) & 3]);                                                          \
@@ -260,7 +260,7 @@ int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *
     StripArgs a;
     a.x = x_dev; a.wq = sp->wq_dev; a.g = sp->g_dev; a.b = sp->b_dev; a.y = y_dev; a.otab = sp->otab_dev;
     a.C = sp->C; a.H = sp->H; a.W = sp->W; a.F = sp->F; a.OW = sp->OW; a.OHW = sp->OH * sp->OW; a.stride = sp->stride; a.pad = sp->pad;
-    a.Kp = sp->Kp; a.Mp = sp->Mp; a.tiles_m = (int)nbl_div_up(sp->F, sp->mt * 32);
+    a.K = sp->K; a.Kp = sp->Kp; a.Mp = sp->Mp; a.tiles_m = (int)nbl_div_up(sp->F, sp->mt * 32);
     a.tiles_per_image = (int)nbl_div_up(a.OHW, STRIP_BN);
     a.rows = sp->rows; a.pitch = sp->pitch; a.act = sp->act;
     a.runs = a.tiles_per_image * (int)B;
