@@ -163,6 +163,63 @@ def test_conv_k_split_matches_oracle_and_unsplit(ctx, case):
     assert rel(got, want) <= TOL
 
 
+def random_conv_case(seed):
+    """A seeded geometry: channel counts either side of the tap-major rule (C % 16 == 0) and of the strip kernel
+    (C <= 4), ragged filter counts, odd and even planes, every cheap activation and one exp-based, and a residual that
+    has the output's shape, fewer channels, more channels, twice the size (read at stride 2), or is absent."""
+    rng = np.random.default_rng(1000 + seed)
+    C = int(rng.choice([1, 3, 4, 5, 8, 16, 24, 32, 48, 64]))
+    k = int(rng.choice([1, 1, 2, 3, 3, 5]))
+    s = int(rng.choice([1, 1, 2]))
+    p = int(rng.integers(0, k // 2 + 2))
+    H, W = int(rng.integers(max(k, 4), 24)), int(rng.integers(max(k, 4), 24))
+    F = int(rng.choice([1, 7, 32, 40, 64, 96, 130, 200]))
+    B = int(rng.integers(1, 5))
+    act = str(rng.choice(["linear", "relu", "leaky", "relie", "logistic"]))
+    post = str(rng.choice(["linear", "relu", "leaky"]))
+    residual = str(rng.choice(["none", "same", "narrow", "wide", "double"]))
+    bn = bool(rng.integers(0, 2))
+    return B, C, H, W, F, k, s, p, bn, act, residual, post
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_conv_random_geometries_every_tile_shape(ctx, seed):
+    from nebula_amd import hip
+    case = random_conv_case(seed)
+    announce("conv random", seed, case)
+    B, Cc, H, W, F, k, s, p, bn, act, residual, post = case
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((B, Cc, H, W)).astype(np.float32)
+    w = (rng.standard_normal((F, Cc, k, k)) * np.sqrt(2.0 / (Cc * k * k))).astype(np.float32)
+    bias = (rng.standard_normal(F) * 0.1).astype(np.float32)
+    bnp = None
+    if bn:
+        bnp = (rng.uniform(0.8, 1.2, F).astype(np.float32), (rng.standard_normal(F) * 0.1).astype(np.float32),
+               rng.uniform(0.5, 1.5, F).astype(np.float32))
+    want = ob.conv_forward(x, w, bias, bnp, s, p, act)
+    OH, OW = want.shape[2:]
+    conn = None
+    if residual != "none":
+        cc = {"same": F, "narrow": max(1, F // 3), "wide": F + 5, "double": max(1, F // 2)}[residual]
+        ch, cw = (2 * OH, 2 * OW) if residual == "double" else (OH, OW)
+        conn = rng.standard_normal((B, cc, ch, cw)).astype(np.float32)
+        want = ob.shortcut_forward(want, conn, post)
+    plan = ctx.conv_pack(w, bias, bnp, H=H, W=W, stride=s, pad=p, act=act)
+    dx = ctx.array(x)
+    dconn = ctx.array(conn) if conn is not None else None
+    run = (lambda: plan.with_shortcut(dx, dconn, post).numpy()) if conn is not None else (lambda: plan(dx).numpy())
+    for v in [-1] + list(range(hip.lib().nbl_conv2d_num_variants())):
+        for split in (0, 1):
+            announce("conv random variant", v, "split", split)
+            plan.set_variant(v)
+            plan.set_split(split if v >= 0 else -1)
+            got = run()
+            assert got.shape == want.shape
+            assert rel(got, want) <= TOL, (case, v, split, rel(got, want))
+            if v < 0:
+                break
+
+
 def test_conv_relu_mask_matches_on_clear_margins(ctx):
     # outputs further than the tolerance from zero must land on the same side of the ReLU
     announce("conv relu mask")
