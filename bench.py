@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # run's tile shapes and k-splits pinned (--dump-launches, then --pin-launches); each counter is scaled by what it reads for
 # `--workload copy` (256 MiB in and out per launch: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Per step: 5203.7 MiB fetched,
 # 2619.6 MiB written over 49 layers.  A recorded measurement, valid for the named workload and batch only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("resnet50", 64): 167.4e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("resnet50", 64): 166.9e6}
 
 
 def log(*a):
