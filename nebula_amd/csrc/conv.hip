@@ -39,31 +39,6 @@ constexpr int CONV_BK = 16;          // k-tile depth (8 MFMA k-steps)
 constexpr int CONV_MP_ALIGN = 384;   // lcm of the BM values below
 constexpr int KTAB_PAD_TAP = 0x4000; // tap row of a padded table entry: always outside the image
 
-// Division by a number known on the host: q = umulhi(n, mul) >> shr for n < 2^31 (mul = ceil(2^(31 + ceil(log2 d)) / d)).
-// A runtime integer division costs some 25 ordinary vector instructions, and the block's set-up has half a dozen of
-// them; ordinary vector instructions are paid for in matrix-pipe time, which matters for layers with few patch rows.
-struct FastDiv {
-    unsigned mul, shr, d;
-    __host__ __device__ __forceinline__ unsigned div(unsigned n) const {
-#if defined(__HIP_DEVICE_COMPILE__)
-        return d == 1u ? n : __umulhi(n, mul) >> shr;
-#else
-        return n / d;
-#endif
-    }
-};
-inline FastDiv make_fastdiv(unsigned d) {
-    FastDiv f; f.d = d; f.mul = 0; f.shr = 0;
-    if(d > 1) {
-        unsigned lg = 0;
-        while((1ull << lg) < d) lg++;
-        const unsigned p = 31 + lg;
-        f.mul = (unsigned)(((1ull << p) + d - 1) / d);
-        f.shr = p - 32;
-    }
-    return f;
-}
-
 struct ConvArgs {
     const float *x; const float *wp; const int2 *ktab; const float *g; const float *b; float *y;
     int H, W, F, OW, OHW, CHW, stride, pad;

@@ -38,6 +38,7 @@ struct StripArgs {
     int rows, pitch;
     int act;
     int runs;               // pixel tiles of the launch (tiles_per_image * batch)
+    FastDiv div_tiles_m, div_tiles_per_image, div_ow;      // the block's set-up divides by these three
 };
 
 // (MT = 2: five blocks per CU fit its LDS use when the registers allow it too -- 6272 tiles of the 7x7 stem at batch 64
@@ -56,15 +57,15 @@ void conv_strip_kernel(const StripArgs a) {
     // (whose strips overlap in all but a row or two) share an XCD, groups of eight are dealt round robin.
     int tm, tn;
     {
-        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = slot / (unsigned)a.tiles_m,
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, run_local = a.div_tiles_m.div(slot),
                        within = slot - run_local * (unsigned)a.tiles_m;
         const unsigned run = ((run_local >> 3) * 8u + xcd) * 8u + (run_local & 7u);
         if(run >= (unsigned)a.runs) return;             // the grid is padded to whole rounds of groups
         tm = (int)within; tn = (int)run;
     }
-    const int img = tn / a.tiles_per_image, p0 = (tn - img * a.tiles_per_image) * STRIP_BN;
+    const int img = (int)a.div_tiles_per_image.div((unsigned)tn), p0 = (tn - img * a.tiles_per_image) * STRIP_BN;
     const int m0 = tm * MT * 32;
-    const int oh0 = p0 / a.OW, ih0 = oh0 * a.stride - a.pad;
+    const int oh0 = (int)a.div_ow.div((unsigned)p0), ih0 = oh0 * a.stride - a.pad;
 
     // ---- stage the strip: rows ih0 .. ih0 + rows - 1, columns -pad .. W + pad - 1 of every channel ----
     // One (channel, row) line per wave at a time, lanes along the line, through a buffer descriptor that covers
@@ -112,7 +113,7 @@ void conv_strip_kernel(const StripArgs a) {
     // this lane's pixel (one per lane: 32 MFMA columns per wave)
     const int pl = p0 + wave * 32 + l32;
     const bool live = pl < a.OHW;
-    const int oh = live ? pl / a.OW : oh0, ow = live ? pl - oh * a.OW : 0;
+    const int oh = live ? (int)a.div_ow.div((unsigned)pl) : oh0, ow = live ? pl - oh * a.OW : 0;
     const int pixbase = (oh - oh0) * a.stride * a.pitch + ow * a.stride;
 
     // weights: lane (half, l32) reads quad 2*s + half of filters m0 + l32*MT + i as 16-byte buffer loads whose
@@ -264,6 +265,8 @@ int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *
     a.tiles_per_image = (int)nbl_div_up(a.OHW, STRIP_BN);
     a.rows = sp->rows; a.pitch = sp->pitch; a.act = sp->act;
     a.runs = a.tiles_per_image * (int)B;
+    a.div_tiles_m = make_fastdiv((unsigned)a.tiles_m); a.div_tiles_per_image = make_fastdiv((unsigned)a.tiles_per_image);
+    a.div_ow = make_fastdiv((unsigned)a.OW);
     const size_t grid = nbl_div_up_sz((size_t)a.runs, 64) * 64 * a.tiles_m;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     const bool fast = sp->act == NBL_ACT_RELU || sp->act == NBL_ACT_LINEAR || sp->act == NBL_ACT_LEAKY || sp->act == NBL_ACT_RELIE;

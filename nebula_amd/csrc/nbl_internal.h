@@ -143,6 +143,31 @@ static inline bool nbl_act_valid(int act) { return act > NBL_ACT_UNDEFINED && ac
 void nbl_fold_batchnorm(const float *bias, const float *scale, const float *mean, const float *var,
                         unsigned n, float *g_out, float *b_out);
 
+// Division by a number known on the host: q = umulhi(n, mul) >> shr for n < 2^31 (mul = ceil(2^(31 + ceil(log2 d)) / d)).
+// A runtime integer division costs some 25 ordinary vector instructions, and the block's set-up has half a dozen of
+// them; ordinary vector instructions are paid for in matrix-pipe time, which matters for layers with few patch rows.
+struct FastDiv {
+    unsigned mul, shr, d;
+    __host__ __device__ __forceinline__ unsigned div(unsigned n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return d == 1u ? n : __umulhi(n, mul) >> shr;
+#else
+        return n / d;
+#endif
+    }
+};
+inline FastDiv make_fastdiv(unsigned d) {
+    FastDiv f; f.d = d; f.mul = 0; f.shr = 0;
+    if(d > 1) {
+        unsigned lg = 0;
+        while((1ull << lg) < d) lg++;
+        const unsigned p = 31 + lg;
+        f.mul = (unsigned)(((1ull << p) + d - 1) / d);
+        f.shr = p - 32;
+    }
+    return f;
+}
+
 // Convolutions with very few input channels (the first layer of an image network: 3 channels, a large filter):
 // their patch rows come from a handful of input rows, so a block stages that strip of the image in LDS once and
 // feeds the matrix cores from it (csrc/conv_strip.hip).  Filled by nbl_conv2d_pack when the layer qualifies.
