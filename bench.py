@@ -233,7 +233,7 @@ def image_input(args):
 
 
 def memory_bound_kernels(args):
-    """The bandwidth-bound kernels at the sizes the BASELINE networks give them, each timed on its own through the C ABI
+    """The bandwidth-bound kernels at the sizes the benchmarked networks (AlexNet, VGG-16, ResNet-50, the LSTM) give them, each timed on its own through the C ABI
     (HIP events on the library's stream, back-to-back launches).  For every kernel: algorithmic bytes per launch (the
     tensors it must read and write once), microseconds per launch and the fraction of the 8 TB/s HBM peak.  The copy
     kernel is the yardstick: what a plain read-once / write-once stream reaches on this machine."""

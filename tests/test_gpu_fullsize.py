@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their real layer shapes.  Against the oracle (OpenBLAS backend, so it
+"""The benchmarked configurations (AlexNet, VGG-16, ResNet-50, the two-layer LSTM) at their real layer shapes.  Against the oracle (OpenBLAS backend, so it
 finishes in seconds) at a batch the CPU can afford, and at the full batch through properties that do
 not depend on size: per-image independence, argmax addressing the maximum, linearity."""
 import numpy as np
