@@ -1182,7 +1182,9 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
 // Tile search on the device: every tile shape, with and without the k-split of the last round, runs the
 // real problem and the fastest wins.  Block-count quantisation against the number of resident blocks
 // decides more than any static rule predicts, so the shapes are measured once per (layer, batch) and the
-// result is kept in the plan.
+// result is kept in the plan.  The first pass splits with the cost model's slice count; the second also tries
+// the other slice counts on the three best tile shapes (the model is off by up to 15 % on some layers: AlexNet's
+// 256 -> 384 3x3 layer at batch 128 takes 351 us with its choice and 300 us with three slices of 128x64 tiles).
 static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
                      const ConvResidual *rs) {
     struct Candidate { int variant; int slices; float ms; };
@@ -1228,15 +1230,44 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
         return NBL_OK;
     };
     if(rc == NBL_OK) rc = pass(cand, 5);
+    size_t ranked = cand.size();          // candidates of the second pass that come from the first
     if(rc == NBL_OK) {
         std::sort(cand.begin(), cand.end(), [](const Candidate &l, const Candidate &r) { return l.ms < r.ms; });
         if(cand.size() > 4) cand.resize(4);
-        rc = pass(cand, 15);
+        ranked = cand.size();
+        if(p->split_mode < 0) {
+            // other slice counts on the best three tile shapes
+            std::vector<int> shapes;
+            for(size_t i = 0; i < cand.size() && shapes.size() < 3; i++)
+                if(cand[i].variant < NUM_VARIANTS && std::find(shapes.begin(), shapes.end(), cand[i].variant) == shapes.end())
+                    shapes.push_back(cand[i].variant);
+            ranked = cand.size();
+            for(int v : shapes) {
+                const Variant &var = VARIANTS[v];
+                const unsigned npix = B * p->OH * p->OW;
+                const int model = plan_split(nbl_div_up(p->F, var.bm), nbl_div_up(npix, var.bn), var.bm, var.bn, p->Kp, p->F, npix, ctx->num_cu, 0).split;
+                for(int g : { 2, 3, 4, 5, 6, 8 }) {
+                    const SplitPlan sp = plan_split(nbl_div_up(p->F, var.bm), nbl_div_up(npix, var.bn), var.bm, var.bn, p->Kp, p->F, npix, ctx->num_cu, g);
+                    if(sp.split != g || g == model) continue;          // fewer patch rows than slices, nothing to split, or measured already
+                    bool have = false;
+                    for(size_t i = 0; i < ranked; i++) have = have || (cand[i].variant == v && cand[i].slices == g);
+                    if(!have) cand.push_back({ v, g, 0.0f });
+                }
+            }
+            ev.resize(cand.size() + 1);
+            for(; made < ev.size(); made++)
+                if(hipEventCreate(&ev[made]) != hipSuccess) { rc = nbl_fail(ctx, NBL_EHIP, "hipEventCreate failed"); break; }
+        }
+        if(rc == NBL_OK) rc = pass(cand, 15);
     }
     for(size_t i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
     if(rc != NBL_OK) return rc;
-    size_t best = 0;
-    for(size_t i = 1; i < cand.size(); i++) if(cand[i].ms < cand[best].ms) best = i;
+    // A slice count the model did not choose has to win by 3 %: with this many candidates the fastest of a pass is
+    // partly the luckiest, and back-to-back launches of one layer are not quite the layer inside its network.
+    size_t best = 0, other = ranked;
+    for(size_t i = 1; i < cand.size() && i < ranked; i++) if(cand[i].ms < cand[best].ms) best = i;
+    for(size_t i = ranked + 1; i < cand.size(); i++) if(cand[i].ms < cand[other].ms) other = i;
+    if(other < cand.size() && cand[other].ms < 0.97f * cand[best].ms) best = other;
     p->tuned_batch = B; p->tuned_variant = cand[best].variant; p->tuned_slices = cand[best].slices;
     return NBL_OK;
 }
