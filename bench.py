@@ -2,16 +2,20 @@
 """Forward-path benchmark.  One step = one forward pass of the workload over one synthetic batch that is
 already resident in HBM.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|alexnet|vgg16|lstm|conv1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|resnet50|alexnet|vgg16|lstm|conv1|...]
 
-Default workload: ResNet-50 (the reference's own topology), fp32, batch 64 -- the configuration the
-headline metric is quoted on.  Besides the throughput the line carries
-  roofline:     the convolution kernel's algorithmic FLOP / its HIP-event time, against the fp32 MFMA peak
+Default (`all`): the headline -- ResNet-50 (the reference's own topology), fp32, batch 64, the configuration the
+metric is quoted on -- timed over K steps, and in the same line, under "configs", the other four benchmarked
+configurations (AlexNet conv1 + pool b32, AlexNet b128, VGG-16 b32, 2-layer LSTM T64 b64) and, under "memops", the
+memory-bound kernels one by one.  Besides the throughput a network's record carries
+  roofline:     the convolution layers' algorithmic FLOP / their HIP-event time, against the fp32 MFMA peak
   cpu_baseline: the reference's CPU algorithm (oracle port, OpenBLAS, all host cores) on a bounded sample.
+`--workload NAME` runs that one workload alone (what the profiles under profiles/ are taken with).
 """
 import argparse
 import json
 import os
+import re
 import sys
 import tempfile
 import time
@@ -21,43 +25,35 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from nebula_amd.zoo import synthetic_weights as make_weights      # noqa: E402
+
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
+# HBM traffic of the convolution layers is a counter measurement (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, over
+# `bench.py --workload NAME`, each scaled by what the same counter reads for `--workload copy`), kept with the
+# profile summary it comes from.  The summary names the launches it was taken with; the figure is reported only
+# when this run's launches are the same.
+TRAFFIC_PROFILES = {("resnet50", 64): os.path.join(ROOT, "profiles", "conv_igemm_resnet50_b64.md")}
 
-# HBM bytes per convolution layer of one step (the layer's kernel plus the finishing kernel of a k-split launch, so the
-# partial sums written and read back are in), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script with the timed
-# run's tile shapes and k-splits pinned (--dump-launches, then --pin-launches); each counter is scaled by what it reads for
-# `--workload copy` (256 MiB in and out per launch: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Per step: 5203.7 MiB fetched,
-# 2619.6 MiB written over 49 layers.  A recorded measurement, valid for the named workload and batch only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("resnet50", 64): 166.9e6}
+
+def measured_traffic(workload_name, batch, conv_tiles):
+    """(bytes per convolution layer, note) from the profile summary of this workload, or (None, why not)."""
+    path = TRAFFIC_PROFILES.get((workload_name, batch))
+    if not path or not os.path.exists(path):
+        return None, "no counter profile of this workload"
+    text = open(path).read()
+    tiles = re.search(r"^conv_tiles: (.*)$", text, re.M)
+    traffic = re.search(r"^traffic_bytes_per_layer: ([0-9.eE+]+)$", text, re.M)
+    if not tiles or not traffic:
+        return None, "the profile summary holds no traffic figure"
+    if tiles.group(1).strip() != conv_tiles.strip():
+        return None, "the counter profile was taken with other launches than this run's"
+    return float(traffic.group(1)), "FETCH_SIZE + WRITE_SIZE of " + os.path.relpath(path, ROOT)
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
-
-
-def make_weights(layout, rng, dist, lstm_hidden=1024):
-    """Synthetic weights in .wgh order from the network's own field table.  dist: 'he' (He-normal weights,
-    N(0,0.01) bias, or for normalised layers beta N(0,0.1), gamma U[0.8,1.2], mean N(0,0.1), var U[0.5,1.5])
-    or 'lstm' (everything U[-1/sqrt(H), 1/sqrt(H)])."""
-    normalised = {li for li, kind, _, _ in layout if kind == "scale"}
-    parts = []
-    for li, kind, count, fan_in in layout:
-        if dist == "lstm":
-            a = rng.uniform(-1, 1, count) / np.sqrt(lstm_hidden)
-        elif kind == "weight":
-            a = rng.standard_normal(count) * np.sqrt(2.0 / fan_in)
-        elif kind == "bias":
-            a = rng.standard_normal(count) * (0.1 if li in normalised else 0.01)
-        elif kind == "scale":
-            a = rng.uniform(0.8, 1.2, count)
-        elif kind == "mean":
-            a = rng.standard_normal(count) * 0.1
-        else:
-            a = rng.uniform(0.5, 1.5, count)
-        parts.append(a.astype(np.float32))
-    return np.concatenate(parts)
 
 
 def workload(name, batch):
@@ -232,7 +228,7 @@ def image_input(args):
     ctx.close()
 
 
-def memory_bound_kernels(args):
+def memory_bound_kernels(args, emit=True):
     """The bandwidth-bound kernels at the sizes the benchmarked networks (AlexNet, VGG-16, ResNet-50, the LSTM) give them, each timed on its own through the C ABI
     (HIP events on the library's stream, back-to-back launches).  For every kernel: algorithmic bytes per launch (the
     tensors it must read and write once), microseconds per launch and the fraction of the 8 TB/s HBM peak.  The copy
@@ -344,6 +340,8 @@ def memory_bound_kernels(args):
     # a kernel that moves less than 64 MB lasts a few microseconds: its figure is launch time, not bandwidth
     for r in out:
         r["launch_bound"] = r["bytes"] < (64 << 20)
+    if not emit:
+        return out
     worst = min(r["frac_of_8TBps"] for r in out[1:] if not r["launch_bound"] and not r.get("matrix_bound"))
     print(json.dumps({"metric": "memory-bound kernels, fraction of the 8 TB/s HBM peak (lowest of the kernels that move 64 MB or more and are not matrix-bound)", "value": worst,
                       "unit": "fraction", "steps": args.steps, "warmup": args.warmup, "peak_GBps": PEAK_HBM_GBS, "kernels": out}), flush=True)
@@ -401,26 +399,226 @@ def recurrent_driver(args):
                       "tokens": out["tokens"], "dense_one_hot": out["dense one-hot"]}), flush=True)
 
 
+CPU_SAMPLES = {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4, "rnn": 4, "dbn": 32, "mlp": 32}
+
+
+def run_network(name, args, steps, warmup, cpu_sample):
+    """Times one network workload and returns its record (the keys of the bench line)."""
+    from nebula_amd import hip
+    from nebula_amd.net import Network
+
+    cfg, batch, xdist, wdist, text = workload(name, args.batch)
+    is_lstm = name in ("lstm", "rnn")        # recurrent: units are sequences, rows are time steps x sequences
+    rng = np.random.default_rng(20240611)
+    if args.launches == "search":
+        hip.lib().nbl_launch_table_clear()          # every convolution problem is measured on the first pass
+    elif args.launches == "model":
+        hip.lib().nbl_launch_table_clear()
+        hip.lib().nbl_launch_table_set_search(0)    # the built-in cost model decides
+    net = Network(cfg)
+    blob = make_weights(net.weight_layout(), rng, wdist)
+    log("workload:", text, "| weights: %.1f MB" % (blob.nbytes / 1e6))
+    with tempfile.NamedTemporaryFile("wb", suffix=".wgh", delete=False) as f:
+        f.write(blob.tobytes())
+        wpath = f.name
+    net.load_weights(wpath)
+    os.unlink(wpath)
+    n_in = net.batch_size * net.input_size
+    x = (rng.random(n_in, dtype=np.float32) if xdist == "uniform" else rng.standard_normal(n_in).astype(np.float32))
+    net.set_input(x)                     # resident in HBM before the timed region
+    del x
+    kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
+    conv_layers = [i for i, k in enumerate(kinds) if k == "convolutional_layer"]
+    if args.pin_launches:
+        pinned = json.load(open(args.pin_launches))
+        assert [p["layer"] for p in pinned] == conv_layers, "--pin-launches: the file lists other layers than this workload has"
+        for p in pinned:
+            net.conv_pin_launch(p["layer"], p["variant"], p["k_slices"] if p["k_slices"] > 1 else 0)
+    use_graph = args.graph == 1
+    if use_graph:
+        net.set_graph(True)              # pass 1 eager, pass 2 recorded, replays from pass 3 (all inside the warm-up)
+        warmup = max(warmup, 3)
+
+    t_first = time.perf_counter()
+    net.forward()
+    net.sync()
+    first_ms = (time.perf_counter() - t_first) * 1e3
+    for _ in range(max(warmup - 1, 0)):
+        net.forward()
+    net.sync()
+    # timed region: K forward passes, synchronised on both sides; HIP events on the library's own stream
+    net.timer_start()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        net.forward()
+    ev_ms = net.timer_stop()
+    net.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+    # what was timed must be a forward pass: finite outputs, and probability rows that sum to one
+    final = net.output(net.num_layers - 1 if kinds[-1] != "cost_layer" else net.num_layers - 2)
+    assert np.isfinite(final).all(), "bench.py: the timed network produced non-finite outputs"
+    if "softmax_layer" in kinds:
+        sm = max(i for i, k in enumerate(kinds) if k == "softmax_layer")
+        rows_out = batch if name == "lstm" else net.batch_size
+        probs = net.output(sm).reshape(net.batch_size, -1)[:rows_out]
+        assert np.abs(probs.sum(1) - 1.0).max() < 1e-3, "bench.py: softmax rows of the timed network do not sum to 1"
+    # tile shape and k slices each convolution launch of the timed passes used, and where the choice came from
+    variant_names = [hip.lib().nbl_conv2d_variant_name(v).decode() for v in range(hip.lib().nbl_conv2d_num_variants() + 1)]
+    launches = []
+    for i in conv_layers:
+        v, g = net.conv_last_launch(i)
+        launches.append({"layer": i, "variant": v, "tile": variant_names[v] if 0 <= v < len(variant_names) else str(v), "k_slices": g,
+                         "source": net.conv_launch_source(i)})
+    if args.dump_launches:
+        with open(args.dump_launches, "w") as f:
+            json.dump(launches, f)
+    sources = sorted({p["source"] for p in launches})
+    conv_tiles = " ".join("%d:%s%s" % (p["layer"], p["tile"], "/%d" % p["k_slices"] if p["k_slices"] > 1 else "") for p in launches)
+    value = batch / (wall / steps)        # images (or sequences) per second
+    log("timed %d steps: wall %.3f ms/step, events %.3f ms/step, first pass %.1f ms" % (steps, ms_per_step, ev_ms / steps, first_ms))
+
+    # HIP events around every layer, in passes of their own over the same network: the layers' shares of a step
+    layer_ms = np.zeros(net.num_layers)
+    reps = max(3, min(10, steps))
+    for _ in range(reps):
+        layer_ms += np.array(net.forward_timed())
+    layer_ms /= reps
+    flops = np.array([net.layer_flop(i) for i in range(net.num_layers)]) * net.batch_size
+    by_kind = {}
+    for k, ms in zip(kinds, layer_ms):
+        by_kind[k] = by_kind.get(k, 0.0) + ms
+    log("per-layer-kind ms:", {k: round(v, 3) for k, v in by_kind.items()})
+    fused = "fuse_shortcut=1" in cfg
+    extra = {}
+    if is_lstm:
+        # per row: 2*(I+H)*4H (lstm), 2*(I+2*O)*O (rnn)
+        rec = [i for i, k in enumerate(kinds) if k in ("lstm_layer", "rnn_layer")]
+        dom_ms = float(layer_ms[rec].sum())
+        steps_per_layer = net.time_step
+        achieved = float(flops[rec].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
+        roofline = {"bound": "mfma", "kernel": "%s_step_kernel" % name,
+                    "covers": "the %d recurrent layers as layers: one input product over all %d time steps (gemm_nt_stream_kernel) and "
+                              "%d dependent step kernels each; HIP events around each layer in passes of their own" % (len(rec), steps_per_layer, steps_per_layer),
+                    "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                    "layers_per_step": len(rec), "avg_layer_ms": round(dom_ms / max(len(rec), 1), 4)}
+    elif name in ("dbn", "mlp"):
+        # weight streaming: every layer reads its [O][I] matrix once per step
+        fc = [i for i, k in enumerate(kinds) if k in ("connected_layer", "rbm_layer")]
+        dom_ms = float(layer_ms[fc].sum())
+        fc_bytes = sum(4.0 * (net.layer_info(i)["input_size"] * net.layer_info(i)["output_size"]
+                              + net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])) for i in fc)
+        gbps = fc_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+        roofline = {"bound": "hbm", "kernel": "gemm_nt_stream_kernel",
+                    "covers": "the %d connected layers as layers (product, split-K reduction, bias, activation); HIP events around each layer in passes of their own" % len(fc),
+                    "achieved": round(gbps, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbps / PEAK_HBM_GBS, 4), "traffic": None,
+                    "layers_per_step": len(fc), "avg_layer_ms": round(dom_ms / max(len(fc), 1), 4),
+                    "algorithmic_bytes_per_layer": round(fc_bytes / max(len(fc), 1)),
+                    "tflops": round(float(flops[fc].sum()) / (dom_ms * 1e-3) / 1e12, 2) if dom_ms > 0 else 0.0}
+    else:
+        conv = conv_layers
+        dom_ms = float(layer_ms[conv].sum())
+        achieved = float(flops[conv].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
+        # the strip kernel takes the layers with very few input channels (index one past the tile shapes)
+        n_strip = sum(1 for p in launches if p["tile"] == "strip")
+        n_finish = sum(1 for p in launches if p["k_slices"] > 1)
+        strip_ms = float(sum(layer_ms[p["layer"]] for p in launches if p["tile"] == "strip"))
+        # algorithmic bytes of the same launches: input + weights + output (+ the residual a fused shortcut reads)
+        algo_bytes = 0.0
+        for i in conv:
+            info = net.layer_info(i)
+            weights = net.layer_flop(i) / (2.0 * info["output_height"] * info["output_width"])
+            residual = info["output_size"] if i + 1 < len(kinds) and kinds[i + 1] == "shortcut_layer" and fused else 0
+            algo_bytes += 4.0 * (net.batch_size * (info["input_size"] + info["output_size"] + residual) + weights)
+        traffic, traffic_note = measured_traffic(name, batch, conv_tiles)
+        roofline = {"bound": "mfma", "kernel": "conv_strip_kernel" if strip_ms > 0.5 * dom_ms else "conv_igemm_kernel",
+                    "covers": "all %d convolution layers as layers: %d conv_igemm_kernel and %d conv_strip_kernel launches plus the %d "
+                              "conv_split_finish_kernel launches behind k-split ones; HIP events around each layer in passes of their own "
+                              "(%d passes, the events' own gaps included)" % (len(conv), len(conv) - n_strip, n_strip, n_finish, reps),
+                    "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                    "traffic": traffic, "traffic_source": traffic_note,
+                    "layers_per_step": len(conv), "avg_layer_ms": round(dom_ms / max(len(conv), 1), 4),
+                    "algorithmic_bytes_per_layer": round(algo_bytes / len(conv)),
+                    "algorithmic_flop_per_layer": round(float(flops[conv].sum()) / len(conv))}
+        # the memory-bound layers of the same step, against the HBM peak: bytes each must read and write once
+        mem = {}
+        for i, k in enumerate(kinds):
+            info = net.layer_info(i)
+            if k in ("maxpool_layer", "avgpool_layer"):
+                mem.setdefault("pooling", [0.0, 0.0])
+                mem["pooling"][0] += 4.0 * net.batch_size * (info["input_size"] + info["output_size"]); mem["pooling"][1] += layer_ms[i]
+            elif k in ("connected_layer", "rbm_layer"):
+                b = 4.0 * (info["input_size"] * info["output_size"] + net.batch_size * (info["input_size"] + info["output_size"]))
+                if 2.0 * net.batch_size * info["input_size"] * info["output_size"] / b <= PEAK_FP32_MFMA_TFLOPS * 1e3 / PEAK_HBM_GBS:
+                    mem.setdefault("connected", [0.0, 0.0])
+                    mem["connected"][0] += b; mem["connected"][1] += layer_ms[i]
+            elif k == "shortcut_layer" and not fused:
+                mem.setdefault("shortcut", [0.0, 0.0])
+                mem["shortcut"][0] += 12.0 * net.batch_size * info["output_size"]; mem["shortcut"][1] += layer_ms[i]
+        extra["memory_bound_layers"] = {k: {"bytes": round(b), "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1) if ms > 0 else 0.0,
+                                            "frac_of_8TBps": round(b / ms / 1e6 / PEAK_HBM_GBS, 3) if ms > 0 else 0.0}
+                                        for k, (b, ms) in mem.items()}
+        if name == "conv1":
+            extra["conv_ms"] = round(float(layer_ms[0]), 4)
+            extra["pool_ms"] = round(float(layer_ms[1]), 4)
+
+    result = {
+        "metric": "ResNet-50 fp32 fwd images/s (bs64, 1 GPU); conv GEMM % of fp32 MFMA peak" if name == "resnet50"
+                  else "%s fp32 fwd %s/s (1 GPU)" % (name, "sequences" if is_lstm else "images"),
+        "value": round(value, 2), "unit": "sequences/s" if is_lstm else "images/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded",
+                   "launch": "hip graph replay" if use_graph and net.graph_active else "eager",
+                   "first_pass_ms": round(first_ms, 1)},
+        "roofline": roofline,
+    }
+    if conv_layers:
+        result["config"]["conv_launches"] = ("pinned from " + os.path.basename(args.pin_launches) if args.pin_launches
+                                             else sources[0] if len(sources) == 1 else "+".join(sources))
+        result["config"]["conv_tiles"] = conv_tiles
+    result.update(extra)
+
+    if cpu_sample != 0:
+        sample = cpu_sample if cpu_sample > 0 else CPU_SAMPLES[name]
+        cfg_fn = (lambda b: workload(name, b)[0])
+        ips, cores, dt, timed, blas, xs, outs = cpu_baseline(cfg_fn, blob, xdist, sample, is_lstm, np.random.default_rng(7))
+        result["cpu_baseline"] = {"value": round(ips, 3), "unit": result["unit"], "cores": cores, "kind": "port",
+                                  "sample": "%d %s of the same workload, %s (%.1f s per forward), %s" % (
+                                      sample, "sequences" if is_lstm else "images",
+                                      "1 timed forward of a fresh network" if timed == 1 else "1 warm-up + mean of %d timed forwards" % timed,
+                                      dt, blas)}
+        log("cpu baseline: %.2f %s on %d cores (%s)" % (ips, result["unit"], cores, blas))
+    net.close()
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "convgrid", "images", "ptb", "memops"],
-                    help="copy: a plain 256 MiB device-to-device copy kernel, the known-size load that HBM traffic "
-                         "counters are calibrated against; conv: one convolution layer (--conv-shape) through the C ABI, "
-                         "for counter passes over a single kernel")
+    ap.add_argument("--workload", default="all", choices=["all", "resnet50", "alexnet", "vgg16", "lstm", "conv1", "rnn", "dbn", "mlp", "copy", "conv", "convgrid", "images", "ptb", "memops"],
+                    help="all (default): the ResNet-50 headline plus the other benchmarked configurations and the memory-bound kernels "
+                         "in one line; a network name: that network alone; copy: a plain 256 MiB device-to-device copy kernel, the "
+                         "known-size load that HBM traffic counters are calibrated against; conv: one convolution layer "
+                         "(--conv-shape) through the C ABI, for counter passes over a single kernel")
     ap.add_argument("--conv-shape", default="512,28,28,256,1,1,0", help="C,H,W,F,k,stride,pad of --workload conv")
-    ap.add_argument("--conv-variant", type=int, default=-1, help="tile shape index of --workload conv (-1: searched)")
-    ap.add_argument("--conv-split", type=int, default=-1, help="k-split mode of --workload conv (-1 searched, 0 off, 1 model)")
+    ap.add_argument("--conv-variant", type=int, default=-1, help="tile shape index of --workload conv (-1: launch table or search)")
+    ap.add_argument("--conv-split", type=int, default=-1, help="k-split mode of --workload conv (-1 launch table or search, 0 off, 1 model)")
     ap.add_argument("--conv-residual", type=int, default=0, help="1: --workload conv adds a same-shape residual and relu in the epilogue (fused shortcut)")
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--recurrent-net", default="lstm", choices=["lstm", "rnn"], help="network of --workload ptb")
+    ap.add_argument("--launches", default="table", choices=["table", "search", "model"],
+                    help="where convolution launches take their tile shape and k-split from: the shipped launch table (problems it does "
+                         "not list are measured on first use), a fresh search of every problem, or the built-in cost model alone")
     ap.add_argument("--dump-launches", default="", help="write the tile shape and k-split every convolution layer ran with (JSON) to this file")
     ap.add_argument("--pin-launches", default="", help="run every convolution layer with the tile shape and k-split listed in this file "
-                    "(as written by --dump-launches) instead of searching: repeats another run's launches exactly, e.g. under counter collection")
+                    "(as written by --dump-launches): repeats another run's launches exactly, e.g. under counter collection")
     ap.add_argument("--graph", type=int, default=0, help="1: forward passes are replays of a recorded HIP graph, 0 (default): eager "
                     "launches (the passes are GPU-bound on this machine: both take the same time)")
     args = ap.parse_args()
@@ -441,150 +639,31 @@ def main():
     if args.workload == "memops":
         return memory_bound_kernels(args)
 
-    from nebula_amd.net import Network
-
-    cfg, batch, xdist, wdist, text = workload(args.workload, args.batch)
-    is_lstm = args.workload in ("lstm", "rnn")        # recurrent: units are sequences, rows are time steps x sequences
-    rng = np.random.default_rng(20240611)
-    net = Network(cfg)
-    blob = make_weights(net.weight_layout(), rng, wdist)
-    log("workload:", text, "| weights: %.1f MB" % (blob.nbytes / 1e6))
-    with tempfile.NamedTemporaryFile("wb", suffix=".wgh", delete=False) as f:
-        f.write(blob.tobytes())
-        wpath = f.name
-    net.load_weights(wpath)
-    os.unlink(wpath)
-    n_in = net.batch_size * net.input_size
-    x = (rng.random(n_in, dtype=np.float32) if xdist == "uniform" else rng.standard_normal(n_in).astype(np.float32))
-    net.set_input(x)                     # resident in HBM before the timed region
-    conv_layers = [i for i in range(net.num_layers) if net.layer_info(i)["kind"] == "convolutional_layer"]
-    if args.pin_launches:
-        pinned = json.load(open(args.pin_launches))
-        assert [p["layer"] for p in pinned] == conv_layers, "--pin-launches: the file lists other layers than this workload has"
-        for p in pinned:
-            net.conv_pin_launch(p["layer"], p["variant"], p["k_slices"] if p["k_slices"] > 1 else 0)
-    use_graph = args.graph == 1
-    if use_graph:
-        net.set_graph(True)              # pass 1 eager, pass 2 recorded, replays from pass 3 (all inside the warm-up)
-        args.warmup = max(args.warmup, 3)
-
-    for _ in range(args.warmup):
-        net.forward()
-    net.sync()
-    # timed region: K forward passes, synchronised on both sides; HIP events on the library's own stream
-    net.timer_start()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        net.forward()
-    ev_ms = net.timer_stop()
-    net.sync()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    # what was timed must be a forward pass: finite outputs, and probability rows that sum to one
-    final = net.output(net.num_layers - 1 if net.layer_info(net.num_layers - 1)["kind"] != "cost_layer" else net.num_layers - 2)
-    assert np.isfinite(final).all(), "bench.py: the timed network produced non-finite outputs"
-    if any(net.layer_info(i)["kind"] == "softmax_layer" for i in range(net.num_layers)):
-        sm = max(i for i in range(net.num_layers) if net.layer_info(i)["kind"] == "softmax_layer")
-        rows_out = batch if (args.workload == "lstm") else net.batch_size
-        probs = net.output(sm).reshape(net.batch_size, -1)[:rows_out]
-        assert np.abs(probs.sum(1) - 1.0).max() < 1e-3, "bench.py: softmax rows of the timed network do not sum to 1"
-    # tile shape and k slices each convolution launch of the timed passes used (searched on the first pass unless pinned)
-    from nebula_amd import hip
-    variant_names = [hip.lib().nbl_conv2d_variant_name(v).decode() for v in range(hip.lib().nbl_conv2d_num_variants() + 1)]
-    launches = []
-    for i in conv_layers:
-        v, g = net.conv_last_launch(i)
-        launches.append({"layer": i, "variant": v, "tile": variant_names[v] if 0 <= v < len(variant_names) else str(v), "k_slices": g})
-    if args.dump_launches:
-        with open(args.dump_launches, "w") as f:
-            json.dump(launches, f)
-    units = batch                         # images (or sequences) per step
-    value = units / (wall / args.steps)
-    log("timed %d steps: wall %.3f ms/step, events %.3f ms/step" % (args.steps, ms_per_step, ev_ms / args.steps))
-
-    # per-layer HIP-event timing over the same workload -> the dominant kernel's achieved rate
-    layer_ms = np.zeros(net.num_layers)
-    reps = max(3, min(10, args.steps))
-    for _ in range(reps):
-        layer_ms += np.array(net.forward_timed())
-    layer_ms /= reps
-    kinds = [net.layer_info(i)["kind"] for i in range(net.num_layers)]
-    flops = np.array([net.layer_flop(i) for i in range(net.num_layers)]) * (net.batch_size if not is_lstm else net.batch_size)
-    by_kind = {}
-    for k, ms in zip(kinds, layer_ms):
-        by_kind[k] = by_kind.get(k, 0.0) + ms
-    log("per-layer-kind ms:", {k: round(v, 3) for k, v in by_kind.items()})
-    algo_bytes = 0.0
-    fused = "fuse_shortcut=1" in cfg
-    roofline = None
-    if is_lstm:
-        # per row: 2*(I+H)*4H (lstm), 2*(I+2*O)*O (rnn)
-        rec = [i for i, k in enumerate(kinds) if k in ("lstm_layer", "rnn_layer")]
-        dom_ms = float(layer_ms[rec].sum())
-        n_launch = len(rec)
-        achieved = float(flops[rec].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
-        dom_name = "%s layers (input product over all steps + one fused kernel per time step)" % args.workload
-    elif args.workload in ("dbn", "mlp"):
-        # weight streaming: every layer reads its [O][I] matrix once per step
-        fc = [i for i, k in enumerate(kinds) if k in ("connected_layer", "rbm_layer")]
-        dom_ms = float(layer_ms[fc].sum())
-        n_launch = len(fc)
-        fc_bytes = sum(4.0 * (net.layer_info(i)["input_size"] * net.layer_info(i)["output_size"]
-                              + net.batch_size * (net.layer_info(i)["input_size"] + net.layer_info(i)["output_size"])) for i in fc)
-        gbps = fc_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
-        roofline = {"bound": "hbm", "kernel": "gemm_nt_kernel (split-K) + splitk_reduce_kernel", "achieved": round(gbps, 1),
-                    "peak": 8000.0, "unit": "GB/s", "frac": round(gbps / 8000.0, 4), "traffic": None,
-                    "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4),
-                    "algorithmic_bytes_per_launch": round(fc_bytes / max(n_launch, 1)),
-                    "tflops": round(float(flops[fc].sum()) / (dom_ms * 1e-3) / 1e12, 2) if dom_ms > 0 else 0.0}
-    else:
-        conv = [i for i, k in enumerate(kinds) if k == "convolutional_layer"]
-        dom_ms = float(layer_ms[conv].sum())
-        n_launch = len(conv)
-        achieved = float(flops[conv].sum()) / (dom_ms * 1e-3) / 1e12 if dom_ms > 0 else 0.0
-        # the strip kernel takes the layers with very few input channels (index one past the tile shapes)
-        strip_ms = float(sum(layer_ms[i] for i in conv if net.conv_last_launch(i)[0] == len(variant_names) - 1))
-        dom_name = "conv_strip_kernel" if strip_ms > 0.5 * dom_ms else "conv_igemm_kernel"
-        # algorithmic bytes of the same launches: input + weights + output (+ the residual a fused shortcut reads)
-        for i in conv:
-            info = net.layer_info(i)
-            weights = net.layer_flop(i) / (2.0 * info["output_height"] * info["output_width"])
-            residual = info["output_size"] if i + 1 < len(kinds) and kinds[i + 1] == "shortcut_layer" and fused else 0
-            algo_bytes += 4.0 * (net.batch_size * (info["input_size"] + info["output_size"] + residual) + weights)
-    if roofline is None:
-        roofline = {"bound": "mfma", "kernel": dom_name, "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, batch)),
-                    "launches_per_step": n_launch, "avg_launch_ms": round(dom_ms / max(n_launch, 1), 4)}
-    if algo_bytes:
-        roofline["algorithmic_bytes_per_launch"] = round(algo_bytes / n_launch)
-        roofline["algorithmic_flop_per_launch"] = round(float(flops[conv].sum()) / n_launch)
-
-    result = {
-        "metric": "ResNet-50 fp32 fwd images/s (bs64, 1 GPU); conv GEMM % of fp32 MFMA peak" if args.workload == "resnet50"
-                  else "%s fp32 fwd %s/s (1 GPU)" % (args.workload, "sequences" if is_lstm else "images"),
-        "value": round(value, 2), "unit": "sequences/s" if is_lstm else "images/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded",
-                   "launch": "hip graph replay" if use_graph and net.graph_active else "eager",
-                   "conv_launches": "pinned from " + os.path.basename(args.pin_launches) if args.pin_launches else "searched on the first pass",
-                   "conv_tiles": " ".join("%d:%s%s" % (p["layer"], p["tile"], "/%d" % p["k_slices"] if p["k_slices"] > 1 else "") for p in launches)},
-        "roofline": roofline,
-    }
-
-    if not args.no_cpu and args.cpu_sample != 0:
-        from nebula_amd import zoo
-        sample = args.cpu_sample if args.cpu_sample > 0 else {"resnet50": 8, "alexnet": 16, "vgg16": 2, "conv1": 32, "lstm": 4, "rnn": 4, "dbn": 32, "mlp": 32}[args.workload]
-        cfg_fn = (lambda b: workload(args.workload, b)[0])
-        ips, cores, dt, timed, blas, xs, outs = cpu_baseline(cfg_fn, blob, xdist, sample, is_lstm, np.random.default_rng(7))
-        result["cpu_baseline"] = {"value": round(ips, 3), "unit": result["unit"], "cores": cores, "kind": "port",
-                                  "sample": "%d %s of the same workload, %s (%.1f s per forward), %s" % (
-                                      sample, "sequences" if is_lstm else "images",
-                                      "1 timed forward of a fresh network" if timed == 1 else "1 warm-up + mean of %d timed forwards" % timed,
-                                      dt, blas)}
-        log("cpu baseline: %.2f %s on %d cores (%s)" % (ips, result["unit"], cores, blas))
-    net.close()
+    cpu = 0 if args.no_cpu else args.cpu_sample
+    if args.workload != "all":
+        print(json.dumps(run_network(args.workload, args, args.steps, args.warmup, cpu)), flush=True)
+        return
+    if args.batch:
+        sys.exit("bench.py: --batch goes with a single --workload")
+    result = run_network("resnet50", args, args.steps, args.warmup, cpu)
+    configs = []
+    for name in ("conv1", "alexnet", "vgg16", "lstm"):
+        r = run_network(name, args, args.steps, args.warmup, cpu)
+        rec = {"workload": r["config"]["workload"], "name": name, "batch": r["config"]["batch"], "ms_per_step": r["ms_per_step"],
+               "value": r["value"], "unit": r["unit"], "steps": r["steps"], "warmup": r["warmup"], "roofline": r["roofline"],
+               "first_pass_ms": r["config"]["first_pass_ms"]}
+        for k in ("conv_launches", "conv_tiles"):
+            if k in r["config"]:
+                rec[k] = r["config"][k]
+        for k in ("memory_bound_layers", "conv_ms", "pool_ms", "cpu_baseline"):
+            if k in r:
+                rec[k] = r[k]
+        configs.append(rec)
+    result["configs"] = configs
+    mem_args = argparse.Namespace(**vars(args))
+    mem_args.steps, mem_args.warmup = min(args.steps, 50), min(max(args.warmup, 3), 10)
+    result["memops"] = [{k: r[k] for k in ("kernel", "bytes", "us", "GBps", "frac_of_8TBps", "launch_bound") if k in r} | ({"matrix_bound": True} if r.get("matrix_bound") else {})
+                        for r in memory_bound_kernels(mem_args, emit=False)]
     print(json.dumps(result), flush=True)
 
 

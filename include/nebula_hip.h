@@ -78,6 +78,11 @@ int nbl_fill_zero(nbl_ctx *ctx, void *dst_dev, size_t bytes);                   
  * layer buffers (models/layers/lstm_layer.cu:41-55, models/layers/connected_layer.cu:244,282). */
 int nbl_copy_d2d(nbl_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 int nbl_sync(nbl_ctx *ctx);
+/* Test support, no counterpart in the reference: overwrites the LDS of (in all likelihood) every CU with a 32-bit
+ * pattern and waits.  LDS keeps what the previous kernel left there, so a kernel that reads LDS words it has not
+ * written itself gives results that depend on its predecessor; running it behind a fill with a NaN pattern
+ * (0x7fc00000, 0xffffffff) makes such a read show in the output. */
+int nbl_lds_fill(nbl_ctx *ctx, unsigned pattern);
 
 /* ---- convolution -------------------------------------------------------------------------------
  * nbl_conv2d_pack replaces convolutional_layer_t::init_weight()'s upload
@@ -133,6 +138,33 @@ int nbl_conv2d_plan_set_split(nbl_conv_plan *plan, int mode);
  * (1 = unsplit) of the plan's most recent launch. */
 int nbl_conv2d_plan_last_launch(const nbl_conv_plan *plan, int *variant, int *split_parts);
 int nbl_conv2d_num_variants(void);
+
+/* ---- launch table --------------------------------------------------------------------------------
+ * The reference's forward is a fixed sequence of library calls (models/networks/network.cc:57-63); here the tile
+ * shape and k-split of a convolution launch are a choice, and the choice is data: a process-wide table keyed by
+ * the problem (C, H, W, F, filter, stride, padding, batch, and the residual a fused shortcut adds: its channels,
+ * height, width and whether the result overwrites it).  On first use the table is read from the text file
+ * <library directory>/../launch_tables/gfx950.txt (the environment variable NBL_LAUNCH_TABLE names another file,
+ * "none" starts empty).  A launch whose plan has neither a pinned tile shape nor a split rule of its own looks
+ * its problem up; a problem the table does not hold is measured on the device once (a few hundred trial launches
+ * that write the real output) and entered, so every later plan of the same problem in the process launches the
+ * same way.  With the search switched off (nbl_launch_table_set_search(0), or NBL_CONV_SEARCH=0 in the
+ * environment) an unlisted problem takes the built-in cost model's choice instead and no launch ever depends on
+ * timing.  Errors of these calls are reported through nbl_last_error(NULL). */
+int nbl_launch_table_load(const char *path);      /* replaces the table with the file's entries (NULL: the default file); returns their number */
+int nbl_launch_table_save(const char *path);      /* writes every entry, read or measured, in the format load reads; returns their number */
+int nbl_launch_table_clear(void);
+int nbl_launch_table_size(void);
+int nbl_launch_table_set_search(int enabled);
+/* Where the plan's most recent launch took its tile shape and k-split from. */
+enum nbl_launch_source {
+    NBL_LAUNCH_NONE = 0,      /* no launch yet */
+    NBL_LAUNCH_PINNED = 1,    /* nbl_conv2d_plan_set_variant */
+    NBL_LAUNCH_TABLE = 2,     /* an entry read from a table file */
+    NBL_LAUNCH_SEARCHED = 3,  /* measured in this process (now, or earlier for an equal problem) */
+    NBL_LAUNCH_MODEL = 4      /* the cost model: tiny problems, or the search switched off */
+};
+int nbl_conv2d_plan_launch_source(const nbl_conv_plan *plan);
 
 /* Replaces _im2col_ (common/utils.h:48, utils.cu:34-74; CPU twin utils.cc:81-119).  The convolution
  * kernel never writes this buffer; the entry point exists so the gather it performs on the fly

@@ -73,7 +73,7 @@ int nbl_net_forward_timed(nbl_net *net, float *ms);
  * it (fuse_shortcut=1) has no buffer of its own: its output is the shortcut's (the sum, activated). */
 int nbl_net_layer_output(nbl_net *net, int layer, float *host, size_t count);
 /* Whose values nbl_net_layer_output(layer) returns after a pass: *writer = layer itself for a layer with a tensor of
- * its own; the [shortcut] behind it for a fused convolution; with shortcut_in_place=1 the last shortcut that wrote its
+ * its own; the producing layer for a [dropout] or [cost] layer (they share its tensor); the [shortcut] behind it for a fused convolution; with shortcut_in_place=1 the last shortcut that wrote its
  * result over this layer's tensor (a ResNet stage then shares one tensor between its blocks and only the last block's
  * output survives the pass). */
 int nbl_net_layer_output_writer(nbl_net *net, int layer, int *writer);
@@ -82,10 +82,17 @@ int nbl_net_layer_output_writer(nbl_net *net, int layer, int *writer);
  * reference ignores); inference never reads the table, so by default it is not written. */
 int nbl_net_pool_index(nbl_net *net, int layer, unsigned *host, size_t count);
 /* Convolutional layers: tile shape index and number of k slices (1 = unsplit) of the layer's most recent launch
- * (nbl_conv2d_plan_last_launch), and a way to pin both (variant < 0: searched on first use; split: -1 searched,
+ * (nbl_conv2d_plan_last_launch), and a way to pin both (variant < 0: from the launch table, or searched on first use; split: -1 likewise,
  * 0 never, 1 cost model, 2..8 that many slices) so that a run can be repeated with exactly the launches of another. */
 int nbl_net_conv_last_launch(nbl_net *net, int layer, int *variant, int *slices);
 int nbl_net_conv_pin_launch(nbl_net *net, int layer, int variant, int split);
+/* Where the layer's most recent launch took its tile shape and k-split from: an nbl_launch_source value of
+ * include/nebula_hip.h (2 = the launch table file, 3 = measured in this process, 1 = pinned, 4 = cost model). */
+int nbl_net_conv_launch_source(nbl_net *net, int layer, int *source);
+/* The launch-table key of a convolutional layer at the network's batch size, twelve numbers in the order of a table
+ * line: C H W F size stride padding batch, then channels, height, width of the residual a fused shortcut adds and 1
+ * when the result is written over it (four zeros without a fused shortcut).  Works on dry-run networks. */
+int nbl_net_conv_problem(nbl_net *net, int layer, unsigned *key);
 /* the softmax layer skips its device->host copy when enabled = 0 (throughput measurement) */
 int nbl_net_softmax_copy(nbl_net *net, int enabled);
 /* enabled = 1 (also the [net] key hip_graph=1, which the reference ignores): nbl_net_forward records the

@@ -21,14 +21,21 @@
 // Work distribution: one block per output tile, except that the tiles of an under-filled last round
 // may be cut into slices along k (one block per slice, raw sums to scratch, a finishing kernel adds
 // them in order and applies the epilogue); block indices are renumbered so that the filter tiles of
-// one pixel tile share an XCD.  The tile shape and whether to split are measured per (layer, batch)
-// on first use.
+// one pixel tile share an XCD.  The tile shape and the k-split of a (layer geometry, batch, residual) come
+// from a launch table: a text file shipped next to the library holds the choices measured for the benchmarked
+// networks, a geometry it does not list is measured on first use (conv_tune) and added to the table in memory,
+// so equal problems launch equally for the life of the process.
 #include "nbl_internal.h"
 
+#include <dlfcn.h>
+
+#include <array>
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
 #include <algorithm>
+#include <map>
+#include <mutex>
 #include <vector>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -892,7 +899,9 @@ struct nbl_conv_plan {
     int2 *ktab_dev; float *g_dev; float *b_dev;
     bool tap_major; int2 *ttab_dev;   // patch rows in (c / 16, i, j, c % 16) order, with a per-k-tile table (C % 16 == 0, 1 < k*k <= 31)
     int variant;   // < 0: chosen per call
-    unsigned tuned_batch; int tuned_variant;   // result of the last on-device tile search
+    unsigned tuned_batch; int tuned_variant;   // the launch chosen for the last (batch, residual) seen: from the table or the tile search
+    std::array<unsigned, 4> tuned_res;         // ... the residual it was chosen for: {channels, height, width, written in place}, zeros without one
+    int launch_source;                         // NBL_LAUNCH_* of the most recent launch
     int split_mode;             // k-split of under-filled launches: -1 measured with the tile search, 0 never, 1 whenever the model below says so, 2..8 always with that many slices
     int tuned_slices;           // 0 = unsplit, 1 = the cost model's slice count, 2..8 = that many
     float *ws_dev; size_t ws_bytes;   // partial sums of split launches (grown on demand)
@@ -954,11 +963,163 @@ SplitPlan plan_split(int tiles_m, int tiles_n, int bm, int bn, unsigned Kp, unsi
     return sp;
 }
 
+
+// ---- launch table --------------------------------------------------------------------------------------------------
+// Which tile shape and how many k slices a convolution launches with is a property of the problem -- geometry, batch,
+// and the residual a fused shortcut adds -- so it is kept in a process-wide table keyed by exactly that.  The table
+// starts from a text file (one line per problem, written by nbl_launch_table_save after a run that measured them);
+// a problem the file does not list is measured once (conv_tune) and entered, so that every later plan of the same
+// problem launches the same way, and nbl_launch_table_save can write the grown table out for the next process.
+//   line:  conv C H W F k stride pad batch res_c res_h res_w in_place tile slices [us]
+//   tile = a name nbl_conv2d_variant_name returns; slices = 0 (unsplit) or 2..8; us = the time measured when the
+//   entry was made (information only).  '#' starts a comment.
+typedef std::array<unsigned, 12> LaunchKey;     // C H W F k stride pad batch res_c res_h res_w in_place
+struct LaunchChoice { int variant; int slices; float us; bool from_file; };
+
+std::mutex g_table_lock;
+std::map<LaunchKey, LaunchChoice> g_table;
+bool g_table_initialised = false;       // the default file has been looked for
+bool g_search_enabled = true;           // problems the table does not list are measured (false: cost model only)
+
+int variant_by_name(const char *name) {
+    for(int v = 0; v < NUM_VARIANTS; v++) if(strcmp(VARIANTS[v].name, name) == 0) return v;
+    return strcmp(name, "strip") == 0 ? NUM_VARIANTS : -1;
+}
+
+// <directory of this shared library>/../launch_tables/gfx950.txt
+std::string default_table_path() {
+    Dl_info info;
+    if(!dladdr((const void*)&variant_by_name, &info) || !info.dli_fname) return std::string();
+    std::string lib(info.dli_fname);
+    const size_t slash = lib.rfind('/');
+    const std::string dir = slash == std::string::npos ? std::string(".") : lib.substr(0, slash);
+    return dir + "/../launch_tables/gfx950.txt";
+}
+
+// Reads a table file into `out`; returns the number of entries or -1 when the file cannot be opened or a line
+// is malformed (`bad_line` then holds its number).
+int read_table_file(const char *path, std::map<LaunchKey, LaunchChoice> &out, int *bad_line) {
+    FILE *f = fopen(path, "r");
+    *bad_line = 0;
+    if(!f) return -1;
+    char line[512];
+    int n = 0, lineno = 0;
+    while(fgets(line, sizeof(line), f)) {
+        lineno++;
+        char *hash = strchr(line, '#');
+        if(hash) *hash = 0;
+        char *q = line;
+        while(*q == ' ' || *q == '\t' || *q == '\n' || *q == '\r') q++;
+        if(!*q) continue;
+        LaunchKey key; char tile[32]; int slices = 0; float us = 0.0f;
+        const int got = sscanf(q, "conv %u %u %u %u %u %u %u %u %u %u %u %u %31s %d %f", &key[0], &key[1], &key[2], &key[3], &key[4],
+                               &key[5], &key[6], &key[7], &key[8], &key[9], &key[10], &key[11], tile, &slices, &us);
+        const int v = got >= 14 ? variant_by_name(tile) : -1;
+        if(got < 14 || v < 0 || slices < 0 || slices == 1 || slices > 8) { *bad_line = lineno; fclose(f); return -1; }
+        LaunchChoice c = { v, slices, got >= 15 ? us : 0.0f, true };
+        out[key] = c;
+        n++;
+    }
+    fclose(f);
+    return n;
+}
+
+// First use: the file NBL_LAUNCH_TABLE names ("none": no file), else the one shipped next to the library.  A file
+// that is missing or malformed leaves the table empty -- every problem is then measured -- and is not an error.
+void table_initialise_locked() {
+    if(g_table_initialised) return;
+    g_table_initialised = true;
+    const char *search = getenv("NBL_CONV_SEARCH");
+    if(search && strcmp(search, "0") == 0) g_search_enabled = false;
+    const char *env = getenv("NBL_LAUNCH_TABLE");
+    if(env && strcmp(env, "none") == 0) return;
+    const std::string path = env && *env ? std::string(env) : default_table_path();
+    if(path.empty()) return;
+    std::map<LaunchKey, LaunchChoice> t;
+    int bad = 0;
+    if(read_table_file(path.c_str(), t, &bad) >= 0) g_table.swap(t);
+}
+
+bool table_lookup(const LaunchKey &key, LaunchChoice *out) {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    const auto it = g_table.find(key);
+    if(it == g_table.end()) return false;
+    *out = it->second;
+    return true;
+}
+
+void table_enter(const LaunchKey &key, const LaunchChoice &c) {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    g_table[key] = c;
+}
+
+bool search_enabled() {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    return g_search_enabled;
+}
+
 }  // namespace
 
 extern "C" {
 
 int nbl_conv2d_num_variants(void) { return NUM_VARIANTS; }
+
+int nbl_launch_table_load(const char *path) {
+    const std::string file = path && *path ? std::string(path) : default_table_path();
+    std::map<LaunchKey, LaunchChoice> t;
+    int bad = 0;
+    const int n = file.empty() ? -1 : read_table_file(file.c_str(), t, &bad);
+    if(n < 0) {
+        if(bad) return nbl_fail(NULL, NBL_EINVAL, "nbl_launch_table_load: %s, line %d: not a launch table line", file.c_str(), bad);
+        return nbl_fail(NULL, NBL_EINVAL, "nbl_launch_table_load: cannot open %s", file.empty() ? "(no default path)" : file.c_str());
+    }
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    g_table_initialised = true;
+    g_table.swap(t);
+    return n;
+}
+
+int nbl_launch_table_clear(void) {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    g_table_initialised = true;
+    g_table.clear();
+    return NBL_OK;
+}
+
+int nbl_launch_table_size(void) {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    return (int)g_table.size();
+}
+
+int nbl_launch_table_save(const char *path) {
+    if(!path || !*path) return nbl_fail(NULL, NBL_EINVAL, "nbl_launch_table_save: no path");
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    FILE *f = fopen(path, "w");
+    if(!f) return nbl_fail(NULL, NBL_EINVAL, "nbl_launch_table_save: cannot write %s", path);
+    fprintf(f, "# gfx950 convolution launch table: tile shape and k slices per problem, as measured on the device\n"
+               "# conv C H W F k stride pad batch res_c res_h res_w in_place tile slices us\n");
+    for(const auto &e : g_table) {
+        fprintf(f, "conv");
+        for(unsigned v : e.first) fprintf(f, " %u", v);
+        fprintf(f, " %s %d %.1f\n", e.second.variant == NUM_VARIANTS ? "strip" : VARIANTS[e.second.variant].name, e.second.slices, e.second.us);
+    }
+    const bool ok = fclose(f) == 0;
+    return ok ? (int)g_table.size() : nbl_fail(NULL, NBL_EINVAL, "nbl_launch_table_save: writing %s failed", path);
+}
+
+int nbl_launch_table_set_search(int enabled) {
+    std::lock_guard<std::mutex> hold(g_table_lock);
+    table_initialise_locked();
+    g_search_enabled = enabled != 0;
+    return NBL_OK;
+}
+
+int nbl_conv2d_plan_launch_source(const nbl_conv_plan *p) { return p ? p->launch_source : NBL_EINVAL; }
 
 const char *nbl_conv2d_variant_name(int variant) {
     return variant == NUM_VARIANTS ? "strip" : variant >= 0 && variant < NUM_VARIANTS ? VARIANTS[variant].name : NULL;
@@ -989,7 +1150,7 @@ int nbl_conv2d_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_ho
     p->Mp = nbl_div_up(F, CONV_MP_ALIGN) * CONV_MP_ALIGN;
     p->act = act; p->has_scale = scale_host != NULL; p->variant = -1;
     p->split_mode = -1; p->tuned_slices = 0; p->ws_dev = NULL; p->ws_bytes = 0; p->last_variant = -1; p->last_split = 1;
-    p->tuned_batch = 0; p->tuned_variant = -1;
+    p->tuned_batch = 0; p->tuned_variant = -1; p->tuned_res = { 0u, 0u, 0u, 0u }; p->launch_source = NBL_LAUNCH_NONE;
     p->strip.eligible = false; p->strip.otab_dev = NULL;
     p->wp_dev = NULL; p->wp_rows_dev = NULL; p->ktab_dev = NULL; p->g_dev = NULL; p->b_dev = NULL; p->ttab_dev = NULL;
     p->tap_major = ksize > 1 && ksize * ksize <= 31 && C % CONV_BK == 0;
@@ -1061,6 +1222,7 @@ int nbl_conv2d_plan_set_variant(nbl_conv_plan *p, int variant) {
     // index NUM_VARIANTS names the strip kernel of layers with very few input channels (only where the plan qualifies)
     if(!p || variant > NUM_VARIANTS || (variant == NUM_VARIANTS && !p->strip.eligible)) return NBL_EINVAL;
     p->variant = variant < 0 ? -1 : variant;
+    p->tuned_batch = 0;
     return NBL_OK;
 }
 
@@ -1186,7 +1348,8 @@ static int conv_launch(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float
 // the other slice counts on the three best tile shapes (the model is off by up to 15 % on some layers: AlexNet's
 // 256 -> 384 3x3 layer at batch 128 takes 351 us with its choice and 300 us with three slices of 128x64 tiles).
 static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
-                     const ConvResidual *rs) {
+                     const ConvResidual *rs, float *winner_us) {
+    *winner_us = 0.0f;
     struct Candidate { int variant; int slices; float ms; };
     std::vector<Candidate> cand;
     for(int v = 0; v < NUM_VARIANTS; v++) {
@@ -1269,40 +1432,120 @@ static int conv_tune(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *
     for(size_t i = ranked + 1; i < cand.size(); i++) if(cand[i].ms < cand[other].ms) other = i;
     if(other < cand.size() && cand[other].ms < 0.97f * cand[best].ms) best = other;
     p->tuned_batch = B; p->tuned_variant = cand[best].variant; p->tuned_slices = cand[best].slices;
+    *winner_us = cand[best].ms * 1000.0f / 15.0f;
     return NBL_OK;
 }
 
-static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B,
-                        const ConvResidual *rs) {
-    nbl_conv_plan *p = const_cast<nbl_conv_plan*>(plan);      // the tile-search result is a cache
-    const size_t in_elems = (size_t)B * p->C * p->H * p->W, out_elems = (size_t)B * p->F * p->OH * p->OW;
+// The search's own measurement of one problem (see conv_tune); y_dev may be the residual itself (in place).
+static int conv_search(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
+                       const ConvResidual *rs, float *winner_us) {
+    if(!(rs && rs->res == y_dev)) return conv_tune(ctx, p, x_dev, y_dev, B, rs, winner_us);
+    // in place: the search's many launches must not feed on their own output, so they write to a buffer of their
+    // own (the residual is only read) and the caller's launch is the one that writes y.  This is the one place
+    // where a forward call holds a second output-sized tensor for a moment; a problem the launch table lists never
+    // comes here.
+    const size_t out_bytes = (size_t)B * p->F * p->OH * p->OW * sizeof(float);
+    float *tmp = NULL;
+    int rc = nbl_malloc(ctx, (void**)&tmp, out_bytes);
+    if(rc != NBL_OK) {
+        const std::string why(ctx->err);
+        return nbl_fail(ctx, rc, "nbl_conv2d_shortcut_fwd: the tile search of an in-place launch needs %zu bytes for its trial outputs (%s); "
+                        "list the problem in the launch table or pin the launch to avoid the search", out_bytes, why.c_str());
+    }
+    rc = conv_tune(ctx, p, x_dev, tmp, B, rs, winner_us);
+    const int rc_free = nbl_free(ctx, tmp);       // waits for the search's launches
+    return rc != NBL_OK ? rc : rc_free;
+}
+
+// One launch (plus the finishing kernel of a k-split one) over B images that fit the kernel's 32-bit offsets.
+static int conv_forward_chunk(nbl_ctx *ctx, nbl_conv_plan *p, const float *x_dev, float *y_dev, unsigned B,
+                              const ConvResidual *rs) {
     const size_t npix = (size_t)B * p->OH * p->OW;
-    if(in_elems >= (1ull << 29) || out_elems >= (1ull << 31) || npix >= (1ull << 31) - 512)
-        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: inputs of 2^29 elements (2 GiB) or more are not supported");
     int v = p->variant;
     int slices = p->split_mode > 0 ? p->split_mode : 0;
-    if(v < 0) {
-        if(p->tuned_batch != B) {
-            // the search overwrites y with correct results several times; tiny problems are not worth it
-            if(2.0 * p->F * p->K * (double)npix < 5e7) { p->tuned_batch = B; p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu); p->tuned_slices = p->split_mode > 0 ? p->split_mode : 0; }
-            else if(rs && rs->res == y_dev) {
-                // in place: the search's many launches must not feed on their own output, so they write to a buffer
-                // of their own (the residual is only read) and the real launch below is the one that writes y
-                float *tmp = NULL;
-                int rc = nbl_malloc(ctx, (void**)&tmp, out_elems * sizeof(float));
+    if(v >= 0) p->launch_source = NBL_LAUNCH_PINNED;
+    else {
+        const std::array<unsigned, 4> res_sig = rs ? std::array<unsigned, 4>{ rs->c, rs->h, rs->w, rs->res == y_dev ? 1u : 0u }
+                                                   : std::array<unsigned, 4>{ 0u, 0u, 0u, 0u };
+        if(p->tuned_batch != B || p->tuned_res != res_sig) {
+            const LaunchKey key = { p->C, p->H, p->W, p->F, p->k, p->stride, p->pad, B, res_sig[0], res_sig[1], res_sig[2], res_sig[3] };
+            LaunchChoice c;
+            // the table holds choices made with everything open; a caller's own split rule is searched under that rule
+            const bool open_split = p->split_mode < 0;
+            const auto usable = [&](const LaunchChoice &lc) {
+                if(lc.variant == NUM_VARIANTS) return p->strip.eligible && !rs;
+                return lc.variant >= 0 && lc.variant < NUM_VARIANTS && nbl_div_up(p->F, VARIANTS[lc.variant].bm) * VARIANTS[lc.variant].bm <= p->Mp;
+            };
+            if(open_split && table_lookup(key, &c) && usable(c)) {
+                p->tuned_variant = c.variant; p->tuned_slices = c.slices;
+                p->launch_source = c.from_file ? NBL_LAUNCH_TABLE : NBL_LAUNCH_SEARCHED;
+            } else if(2.0 * p->F * p->K * (double)npix < 5e7 || !search_enabled()) {
+                // the search overwrites y with correct results several times; tiny problems are not worth it
+                p->tuned_variant = choose_variant(p, (unsigned)npix, ctx->num_cu);
+                p->tuned_slices = p->split_mode > 0 ? p->split_mode : p->split_mode < 0 && 2.0 * p->F * p->K * (double)npix >= 5e7 ? 1 : 0;
+                p->launch_source = NBL_LAUNCH_MODEL;
+            } else {
+                float us = 0.0f;
+                const int rc = conv_search(ctx, p, x_dev, y_dev, B, rs, &us);
                 if(rc != NBL_OK) return rc;
-                rc = conv_tune(ctx, p, x_dev, tmp, B, rs);
-                const int rc_free = nbl_free(ctx, tmp);       // waits for the search's launches
-                if(rc != NBL_OK) return rc;
-                if(rc_free != NBL_OK) return rc_free;
+                p->launch_source = NBL_LAUNCH_SEARCHED;
+                if(open_split) {
+                    // entered with the slice count written out (1 stands for "what the cost model says")
+                    int written = p->tuned_slices;
+                    if(written == 1 && p->tuned_variant < NUM_VARIANTS) {
+                        const Variant &var = VARIANTS[p->tuned_variant];
+                        const int model = plan_split(nbl_div_up(p->F, var.bm), nbl_div_up((unsigned)npix, var.bn), var.bm, var.bn,
+                                                     p->Kp, p->F, (unsigned)npix, ctx->num_cu, 0).split;
+                        written = model > 1 ? model : 0;
+                    }
+                    const LaunchChoice found = { p->tuned_variant, written, us, false };
+                    table_enter(key, found);
+                    p->tuned_slices = written;
+                }
             }
-            else { int rc = conv_tune(ctx, p, x_dev, y_dev, B, rs); if(rc != NBL_OK) return rc; }
+            p->tuned_batch = B; p->tuned_res = res_sig;
         }
         v = p->tuned_variant;
         slices = p->tuned_slices;
     }
     if(v == NUM_VARIANTS && rs) { v = choose_variant(p, (unsigned)npix, ctx->num_cu); slices = 0; }     // the strip kernel fuses no shortcut
     return conv_launch(ctx, p, x_dev, y_dev, B, v, slices, rs);
+}
+
+// Images per launch: the kernels address the input with 32-bit byte offsets (below 2^31, the top bit marks an
+// out-of-range lane), the output and the residual with 32-bit element counts.  A larger batch runs as consecutive
+// slices of whole images, each its own launch with its own table entry -- images are independent, as in the
+// reference's per-image loop (models/layers/convolutional_layer.cc:374-399).
+static unsigned conv_images_per_launch(const nbl_conv_plan *p, const ConvResidual *rs) {
+    const size_t in_image = (size_t)p->C * p->H * p->W, out_image = (size_t)p->F * p->OH * p->OW;
+    const size_t res_image = rs ? (size_t)rs->c * rs->h * rs->w : 0;
+    size_t n = (((size_t)1 << 29) - 1) / in_image;
+    n = std::min<size_t>(n, (((size_t)1 << 31) - 1) / out_image);
+    n = std::min<size_t>(n, (((size_t)1 << 31) - 1024) / ((size_t)p->OH * p->OW));
+    if(res_image) n = std::min<size_t>(n, (((size_t)1 << 31) - 1) / res_image);
+    return (unsigned)std::min<size_t>(n, 0xffffffffu);
+}
+
+static int conv_forward(nbl_ctx *ctx, const nbl_conv_plan *plan, const float *x_dev, float *y_dev, unsigned B,
+                        const ConvResidual *rs) {
+    nbl_conv_plan *p = const_cast<nbl_conv_plan*>(plan);      // the chosen launch is a cache
+    const unsigned per_launch = conv_images_per_launch(p, rs);
+    if(per_launch == 0)
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: one image of this layer has 2^29 input or 2^31 output elements or more");
+    if(B <= per_launch) return conv_forward_chunk(ctx, p, x_dev, y_dev, B, rs);
+    // equal slices rather than full ones and a remainder: at most two batch sizes, hence two table entries, ever occur
+    const unsigned launches = nbl_div_up(B, per_launch), base = B / launches, extra = B % launches;
+    const size_t in_image = (size_t)p->C * p->H * p->W, out_image = (size_t)p->F * p->OH * p->OW;
+    unsigned done = 0;
+    for(unsigned i = 0; i < launches; i++) {
+        const unsigned nb = base + (i < extra ? 1u : 0u);
+        ConvResidual part;
+        if(rs) { part = *rs; part.res = rs->res + (size_t)done * rs->c * rs->h * rs->w; }
+        const int rc = conv_forward_chunk(ctx, p, x_dev + (size_t)done * in_image, y_dev + (size_t)done * out_image, nb, rs ? &part : NULL);
+        if(rc != NBL_OK) return rc;
+        done += nb;
+    }
+    return NBL_OK;
 }
 
 // [a, a + a_bytes) and [b, b + b_bytes) share a byte
@@ -1341,8 +1584,6 @@ int nbl_conv2d_shortcut_fwd(nbl_ctx *ctx, const nbl_conv_plan *plan, const float
                 "nbl_conv2d_shortcut_fwd: y must not overlap x");
     if(plan->OW / conn_w > 1)
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: an up-sampling shortcut cannot be fused");
-    if((size_t)B * conn_c * conn_h * conn_w >= (1ull << 31))
-        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_shortcut_fwd: residual tensor too large");
     if(B == 0) return NBL_OK;
     ConvResidual rs = { conn_dev, conn_c, conn_h, conn_w, post_act };
     return conv_forward(ctx, plan, x_dev, y_dev, B, &rs);

@@ -48,8 +48,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MT == 2 ? 5
 void conv_strip_kernel(const StripArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int strip_elems = a.C * a.rows * a.pitch;
-    float *strip = lds;                                     // [C][rows][pitch], then 4 zero floats
-    int *otab = reinterpret_cast<int*>(lds + ((strip_elems + 4 + 3) & ~3));     // [Kp], 16-byte aligned
+    float *strip = lds;                                     // [C][rows][pitch]
+    int *otab = reinterpret_cast<int*>(lds + ((strip_elems + 3) & ~3));         // [Kp], 16-byte aligned
 
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // uniform, and known to be: per-row buffer descriptors are built from it
@@ -105,7 +105,6 @@ void conv_strip_kernel(const StripArgs a) {
                 }
             }
         }
-        if(tid < 4) strip[strip_elems + tid] = 0.0f;        // what padding rows of the patch matrix read
         for(int e = tid; e < a.Kp; e += 256) otab[e] = a.otab[e];
     }
     __syncthreads();
@@ -121,7 +120,10 @@ void conv_strip_kernel(const StripArgs a) {
     const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.wq), 0, (int)((unsigned)a.Kp * (unsigned)a.Mp * 4u), 0x00020000);
     const unsigned w_lane = (unsigned)(half * a.Mp + m0 + l32 * MT) * 16u;
     const unsigned w_step = (unsigned)a.Mp * 32u;           // two quads of k per step
-    const int nsteps = (a.K + 7) / 8;     // steps of 8 patch rows; the packed weights are zero from row K to row Kp
+    // steps of 8 patch rows; the packed weights are zero from row K to row Kp, and the table sends those rows to strip
+    // offset 0, so that they read the pixel's own first tap (initialised image data) against the zero weight and never
+    // a word of LDS this block has not written
+    const int nsteps = (a.K + 7) / 8;
     auto load_a = [&](vec4f (&dst)[MT], int s) {
         #pragma unroll
         for(int i = 0; i < MT; i++)
@@ -232,11 +234,14 @@ int nbl_conv_strip_pack(nbl_ctx *ctx, nbl_strip_plan *sp) {
     sp->rows = (rows_out - 1) * sp->stride + sp->k;
     sp->pitch = sp->W + 2 * sp->pad;
     const size_t strip_elems = (size_t)sp->C * sp->rows * sp->pitch;
-    sp->lds_bytes = ((strip_elems + 4 + 3) & ~(size_t)3) * sizeof(float) + (size_t)sp->Kp * sizeof(int);
+    sp->lds_bytes = ((strip_elems + 3) & ~(size_t)3) * sizeof(float) + (size_t)sp->Kp * sizeof(int);
     if(sp->lds_bytes > STRIP_LDS_LIMIT) return NBL_OK;
     sp->mt = sp->F <= 64 ? 2 : sp->F <= 96 ? 3 : 4;
     if((unsigned)(nbl_div_up(sp->F, sp->mt * 32) * sp->mt * 32) > (unsigned)sp->Mp) return NBL_OK;   // the last filter tile must exist in the packed weights
-    std::vector<int> otab(sp->Kp, (int)strip_elems);       // padding rows read the zero word behind the strip
+    // padding rows (K .. Kp) get offset 0: added to a pixel's base that is the pixel's first tap of channel 0, a word the
+    // block has staged; its product with the zero weight of a padding row is 0 (or NaN exactly where the real
+    // patch holds a NaN or Inf in that tap, which makes the sum NaN already)
+    std::vector<int> otab(sp->Kp, 0);
     for(int c = 0; c < sp->C; c++)
         for(int i = 0; i < sp->k; i++)
             for(int j = 0; j < sp->k; j++)

@@ -60,6 +60,13 @@ int nbl_ctx_create_on_stream(int device, void *hip_stream, nbl_ctx **out) {
         delete ctx;
         return nbl_fail(NULL, NBL_EHIP, "hipEventCreate: %s", hipGetErrorString(e));
     }
+    const int rc = nbl_fc_scratch_resolve(ctx);
+    if(rc != NBL_OK) {
+        nbl_fail(NULL, rc, "%s", ctx->err);
+        (void)hipEventDestroy(ctx->ev_start); (void)hipEventDestroy(ctx->ev_stop);
+        delete ctx;
+        return rc;
+    }
     *out = ctx;
     return NBL_OK;
 }
@@ -218,6 +225,34 @@ int nbl_copy_d2d(nbl_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes)
                            (unsigned char*)dst_dev + n4 * 16, (const unsigned char*)src_dev + n4 * 16, ntail);
     NBL_LAUNCH_CHECK(ctx, "copy_d2d");
     return NBL_OK;
+}
+
+// Every block writes `words` 32-bit words of its LDS allocation with the pattern and reports one of them, so the
+// stores cannot be dropped.
+__global__ void nbl_lds_fill_kernel(unsigned pattern, unsigned words, unsigned *sink) {
+    extern __shared__ unsigned lds_words[];
+    for(unsigned i = threadIdx.x; i < words; i += blockDim.x) lds_words[i] = pattern;
+    __syncthreads();
+    if(threadIdx.x == 0 && lds_words[words - 1] != pattern) *sink = 1u;
+}
+
+int nbl_lds_fill(nbl_ctx *ctx, unsigned pattern) {
+    if(!ctx) return NBL_EINVAL;
+    int max_bytes = 0;
+    NBL_HIP(ctx, hipDeviceGetAttribute(&max_bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, ctx->device));
+    if(max_bytes <= 0) return nbl_fail(ctx, NBL_EHIP, "nbl_lds_fill: the device reports no LDS");
+    if(max_bytes > 64 * 1024)
+        NBL_HIP(ctx, hipFuncSetAttribute((const void*)nbl_lds_fill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_bytes));
+    unsigned *sink = NULL;
+    int rc = nbl_malloc(ctx, (void**)&sink, sizeof(unsigned));
+    if(rc != NBL_OK) return rc;
+    // a block takes a CU's whole LDS, so at most one is resident per CU; a few rounds reach every CU
+    hipLaunchKernelGGL(nbl_lds_fill_kernel, dim3(8u * (unsigned)ctx->num_cu), dim3(256), (size_t)max_bytes, ctx->stream,
+                       pattern, (unsigned)max_bytes / 4u, sink);
+    hipError_t e = hipGetLastError();
+    rc = nbl_free(ctx, sink);       // waits for the kernel
+    if(e != hipSuccess) return nbl_fail(ctx, NBL_EHIP, "launch of nbl_lds_fill_kernel failed: %s", hipGetErrorString(e));
+    return rc;
 }
 
 int nbl_sync(nbl_ctx *ctx) {

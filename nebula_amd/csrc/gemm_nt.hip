@@ -934,7 +934,7 @@ int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float 
 // ---- fully connected without allocation ----------------------------------------------------------
 // Split-K partial sums of nbl_fc_fwd_noalloc live in a file-scope device array, one copy per GPU for the life of
 // the process.  On the host the array's NAME is only a handle: the address kernels can use comes from
-// hipGetSymbolAddress, asked once per device with that device current, and is kept per device.
+// hipGetSymbolAddress, asked once per device with that device current (at context creation), and is kept per device.
 }  // extern "C"
 
 namespace {
@@ -945,24 +945,26 @@ static __device__ __align__(256) float fc_noalloc_scratch[FC_SCRATCH_BYTES / siz
 float *g_fc_scratch_ptr[FC_SCRATCH_MAX_DEVICES];
 std::mutex g_fc_scratch_lock;
 
-// Device address of this GPU's copy of the scratch array (looked up on the first call for the device).
-int fc_scratch_address(nbl_ctx *ctx, float **out) {
-    if(ctx->device < 0 || ctx->device >= FC_SCRATCH_MAX_DEVICES)
-        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: device index %d beyond %d", ctx->device, FC_SCRATCH_MAX_DEVICES);
+}  // namespace
+
+// Device address of this GPU's copy of the scratch array, looked up once per device (with that device current) when
+// the device's first context is created, so that nbl_fc_fwd_noalloc itself only launches kernels -- nothing in it
+// loads a code object or touches the current device, which a stream capture around it could not record.
+int nbl_fc_scratch_resolve(nbl_ctx *ctx) {
+    ctx->fc_scratch = NULL;
+    if(ctx->device < 0 || ctx->device >= FC_SCRATCH_MAX_DEVICES) return NBL_OK;      // nbl_fc_fwd_noalloc refuses such a context
     std::lock_guard<std::mutex> hold(g_fc_scratch_lock);
     if(!g_fc_scratch_ptr[ctx->device]) {
         NBL_HIP(ctx, hipSetDevice(ctx->device));
         void *p = NULL;
         NBL_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(fc_noalloc_scratch)));
         if(!p || ((size_t)p & 255) != 0)
-            return nbl_fail(ctx, NBL_EHIP, "nbl_fc_fwd_noalloc: hipGetSymbolAddress returned an unusable address %p", p);
+            return nbl_fail(ctx, NBL_EHIP, "hipGetSymbolAddress returned an unusable address %p for the static scratch array", p);
         g_fc_scratch_ptr[ctx->device] = (float*)p;
     }
-    *out = g_fc_scratch_ptr[ctx->device];
+    ctx->fc_scratch = g_fc_scratch_ptr[ctx->device];
     return NBL_OK;
 }
-
-}  // namespace
 
 extern "C" {
 
@@ -972,9 +974,9 @@ int nbl_fc_fwd_noalloc(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev
     if(B == 0) return NBL_OK;
     if((size_t)B * plan->I >= (1ull << 31) || (size_t)B * plan->O >= (1ull << 31))
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: tensors of 2^31 elements or more are not supported");
-    float *scratch = NULL;
-    const int rc = fc_scratch_address(ctx, &scratch);
-    if(rc != NBL_OK) return rc;
+    float *scratch = ctx->fc_scratch;
+    if(!scratch)
+        return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: no static scratch on device %d (index beyond %d)", ctx->device, FC_SCRATCH_MAX_DEVICES);
     // every partial sum the reduction reads is written by this call's product kernel first, so the contents a
     // previous call left behind never show
     return launch_fc(ctx, x_dev, plan->w_dev, y_dev, (int)B, (int)plan->O, (int)plan->I, plan->g_dev, plan->b_dev,

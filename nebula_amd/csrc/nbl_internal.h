@@ -20,7 +20,11 @@ struct nbl_ctx {
     // tap tables of the last image resize geometry (nbl_image_to_input), kept on the device
     unsigned rz_src_h, rz_src_w, rz_dst_h, rz_dst_w;
     int *rz_tab_dev;
+    float *fc_scratch;      // this device's copy of the static split-K scratch of nbl_fc_fwd_noalloc (NULL: none)
 };
+
+// Looks up the device address of the static scratch array for ctx->device (once per device) and stores it in the context.
+int nbl_fc_scratch_resolve(nbl_ctx *ctx);
 
 // Records a formatted message on the context and returns `code`.
 int nbl_fail(nbl_ctx *ctx, int code, const char *fmt, ...);
@@ -176,7 +180,7 @@ struct nbl_strip_plan {
     int C, H, W, F, k, stride, pad, OH, OW, K, Kp, Mp, act;
     int mt;                 // 32-filter MFMA tiles per wave (block tile = 32*mt filters x 128 pixels)
     int rows, pitch;        // strip: input rows a block may need, floats per row (W + 2*pad)
-    int *otab_dev;          // [Kp] strip offset of every patch row; padding rows point at a zero word behind the strip
+    int *otab_dev;          // [Kp] strip offset of every patch row; padding rows hold 0 (the pixel's own first tap, against a zero weight)
     const float *wq_dev, *g_dev, *b_dev;     // packed weights [Kp / 4][Mp][4], per-filter multiply-add
     size_t lds_bytes;
 };

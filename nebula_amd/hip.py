@@ -15,6 +15,7 @@ ACT_NAMES = ["undefined_activation", "elu", "hardtan", "leaky", "lhtan", "linear
              "plse", "ramp", "relie", "relu", "stair", "tanh"]
 ACT = {n: i for i, n in enumerate(ACT_NAMES)}
 POOL_MAX, POOL_AVG = 0, 1
+LAUNCH_SOURCES = ["none", "pinned", "table", "searched", "model"]      # enum nbl_launch_source
 
 _vp = C.c_void_p
 _u = C.c_uint
@@ -38,6 +39,13 @@ SIGNATURES = {
     "nbl_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
     "nbl_copy_d2d": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "nbl_sync": (C.c_int, [_vp]),
+    "nbl_lds_fill": (C.c_int, [_vp, _u]),
+    "nbl_launch_table_load": (C.c_int, [C.c_char_p]),
+    "nbl_launch_table_save": (C.c_int, [C.c_char_p]),
+    "nbl_launch_table_clear": (C.c_int, []),
+    "nbl_launch_table_size": (C.c_int, []),
+    "nbl_launch_table_set_search": (C.c_int, [C.c_int]),
+    "nbl_conv2d_plan_launch_source": (C.c_int, [_vp]),
     "nbl_lstm_fwd_tokens": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
     "nbl_rnn_pack": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_rnn_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u]),
@@ -350,6 +358,9 @@ class ConvPlan:
         v, g = C.c_int(), C.c_int()
         self.ctx.check(lib().nbl_conv2d_plan_last_launch(self.p, C.byref(v), C.byref(g)))
         return v.value, g.value
+
+    def launch_source(self):
+        return LAUNCH_SOURCES[lib().nbl_conv2d_plan_launch_source(self.p)]
 
     def set_split(self, mode):
         """-1: measured on first use, 0: never split along k, 1: split wherever the cost model says so, 2..8: that many slices."""

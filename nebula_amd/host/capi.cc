@@ -169,8 +169,11 @@ int nbl_net_layer_output_writer(nbl_net *n, int i, int *writer) {
         if(!writer) throw std::runtime_error("Error: writer is NULL");
         // the last layer with a kernel of its own that writes the tensor this layer's output pointer refers to
         (void)l;
-        *writer = i;
         const std::vector<layer_t*> &layers = n->net->layers;
+        // a dropout or cost layer has no kernel: its values are its producer's
+        int own = i;
+        while(own > 0 && (layers[own]->layer_type == DROPOUT_LAYER || layers[own]->layer_type == COST_LAYER)) own--;
+        *writer = own;
         const std::vector<int> &tensor = n->net->output_tensor;
         for(int j = i + 1; j < (int)layers.size() && j < (int)tensor.size(); j++) {
             const layer_type_t t = layers[j]->layer_type;
@@ -194,6 +197,30 @@ int nbl_net_conv_last_launch(nbl_net *n, int i, int *variant, int *slices) {
         layer_t *l = layer_at(n, i);
         if(l->layer_type != CONVOLUTIONAL_LAYER) throw std::runtime_error("Error: not a convolutional layer");
         static_cast<convolutional_layer_t*>(l)->last_launch(variant, slices));
+}
+
+int nbl_net_conv_problem(nbl_net *n, int i, unsigned *key) {
+    NBL_NET_TRY(
+        layer_t *l = layer_at(n, i);
+        if(l->layer_type != CONVOLUTIONAL_LAYER) throw std::runtime_error("Error: not a convolutional layer");
+        if(!key) throw std::runtime_error("Error: key is NULL");
+        const convolutional_layer_t *c = static_cast<convolutional_layer_t*>(l);
+        key[0] = c->input_channel; key[1] = c->input_height; key[2] = c->input_width; key[3] = c->num_filters;
+        key[4] = c->filter_size; key[5] = c->stride; key[6] = c->padding; key[7] = n->net->batch_size;
+        key[8] = key[9] = key[10] = key[11] = 0;
+        if(c->shortcut_fused()) {
+            const layer_t *conn = c->shortcut_fused()->connection;
+            key[8] = conn->output_channel; key[9] = conn->output_height; key[10] = conn->output_width;
+            key[11] = c->shortcut_fused()->in_place ? 1u : 0u;
+        });
+}
+
+int nbl_net_conv_launch_source(nbl_net *n, int i, int *source) {
+    NBL_NET_TRY(
+        layer_t *l = layer_at(n, i);
+        if(l->layer_type != CONVOLUTIONAL_LAYER) throw std::runtime_error("Error: not a convolutional layer");
+        if(!source) throw std::runtime_error("Error: source is NULL");
+        *source = static_cast<convolutional_layer_t*>(l)->launch_source());
 }
 
 int nbl_net_conv_pin_launch(nbl_net *n, int i, int variant, int split) {

@@ -192,6 +192,11 @@ void convolutional_layer_t::last_launch(int *variant, int *slices) const {
     nbl_check(network->ctx, nbl_conv2d_plan_last_launch(plan, variant, slices), "nbl_conv2d_plan_last_launch");
 }
 
+int convolutional_layer_t::launch_source() const {
+    if(!plan) throw std::runtime_error("Error: convolutional layer has no weights (init_weight not called)");
+    return nbl_conv2d_plan_launch_source(plan);
+}
+
 void convolutional_layer_t::pin_launch(int variant, int split) {
     if(!plan) throw std::runtime_error("Error: convolutional layer has no weights (init_weight not called)");
     nbl_check(network->ctx, nbl_conv2d_plan_set_variant(plan, variant), "nbl_conv2d_plan_set_variant");

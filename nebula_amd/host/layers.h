@@ -84,10 +84,12 @@ public:
     // be fused (up-sampling shortcut, or a shortcut whose source is this very layer).
     bool fuse_with(class shortcut_layer_t *m_shortcut);
     // Tile shape and k-split of the kernel: what the most recent forward used, and a way to pin both
-    // (variant < 0: searched on first use; split as nbl_conv2d_plan_set_split).
+    // (variant < 0: from the launch table, or searched on first use; split as nbl_conv2d_plan_set_split).
     void last_launch(int *variant, int *slices) const;
+    int launch_source() const;          // nbl_launch_source of the most recent launch
     void pin_launch(int variant, int split);
     bool is_fused() const { return fused_shortcut != NULL; }
+    const class shortcut_layer_t *shortcut_fused() const { return fused_shortcut; }
 private:
     void pack();
     bool batch_normalize;

@@ -208,6 +208,11 @@ void inference_net_t::build(config_t &config) {
             if(safe) sc->write_over_connection();
         }
     }
+    // Dropout and cost layers copied their producer's output pointer when they were initialised; a fusion or an in-place
+    // shortcut above has since freed or replaced some of those tensors, so every alias is taken again, in layer order.
+    for(unsigned i = 1; i < num_layers; i++)
+        if(layers[i]->layer_type == DROPOUT_LAYER || layers[i]->layer_type == COST_LAYER)
+            layers[i]->output_data_dev = layers[i - 1]->output_data_dev;
     // Which tensor every layer's output pointer refers to (the index of the layer that owns it): dropout and cost layers
     // share their producer's, a fused convolution its shortcut's, an in-place shortcut its connection's.
     output_tensor.assign(num_layers, 0);

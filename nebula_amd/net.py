@@ -38,6 +38,8 @@ SIGNATURES = {
     "nbl_net_pool_index": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t]),
     "nbl_net_conv_last_launch": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "nbl_net_conv_pin_launch": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int]),
+    "nbl_net_conv_launch_source": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_int)]),
+    "nbl_net_conv_problem": (C.c_int, [_vp, C.c_int, C.POINTER(_u)]),
     "nbl_net_softmax_copy": (C.c_int, [_vp, C.c_int]),
     "nbl_net_set_graph": (C.c_int, [_vp, C.c_int]),
     "nbl_net_graph_active": (C.c_int, [_vp]),
@@ -193,6 +195,18 @@ class Network:
         v, g = C.c_int(), C.c_int()
         self._check(lib().nbl_net_conv_last_launch(self.h, i, C.byref(v), C.byref(g)))
         return v.value, g.value
+
+    def conv_problem(self, i):
+        """Launch-table key of convolutional layer i: (C, H, W, F, size, stride, padding, batch, res_c, res_h, res_w, in_place)."""
+        key = (_u * 12)()
+        self._check(lib().nbl_net_conv_problem(self.h, i, key))
+        return tuple(key)
+
+    def conv_launch_source(self, i):
+        """Where layer i's most recent launch took its tile shape from: one of hip.LAUNCH_SOURCES."""
+        v = C.c_int()
+        self._check(lib().nbl_net_conv_launch_source(self.h, i, C.byref(v)))
+        return hip.LAUNCH_SOURCES[v.value]
 
     def conv_pin_launch(self, i, variant, split):
         """Pin layer i's tile shape (variant < 0: searched) and k-split (-1 searched, 0 never, 1 cost model, 2..8 slices)."""

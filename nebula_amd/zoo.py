@@ -115,6 +115,30 @@ def mlp_cfg(batch=32):
     return s
 
 
+def synthetic_weights(layout, rng, dist, lstm_hidden=1024):
+    """Synthetic weights in .wgh order from a network's own field table (Network.weight_layout()).  dist: 'he'
+    (He-normal weights, N(0,0.01) bias, or for normalised layers beta N(0,0.1), gamma U[0.8,1.2], mean N(0,0.1),
+    var U[0.5,1.5]) or 'lstm' (everything U[-1/sqrt(H), 1/sqrt(H)])."""
+    import numpy as np
+    normalised = {li for li, kind, _, _ in layout if kind == "scale"}
+    parts = []
+    for li, kind, count, fan_in in layout:
+        if dist == "lstm":
+            a = rng.uniform(-1, 1, count) / np.sqrt(lstm_hidden)
+        elif kind == "weight":
+            a = rng.standard_normal(count) * np.sqrt(2.0 / fan_in)
+        elif kind == "bias":
+            a = rng.standard_normal(count) * (0.1 if li in normalised else 0.01)
+        elif kind == "scale":
+            a = rng.uniform(0.8, 1.2, count)
+        elif kind == "mean":
+            a = rng.standard_normal(count) * 0.1
+        else:
+            a = rng.uniform(0.5, 1.5, count)
+        parts.append(a.astype(np.float32))
+    return np.concatenate(parts)
+
+
 WORKLOADS = {
     "conv1": conv1_pool_cfg, "alexnet": alexnet_cfg, "vgg16": vgg16_cfg, "resnet50": resnet50_cfg, "lstm": lstm_cfg,
     "rnn": rnn_cfg, "dbn": dbn_cfg, "mlp": mlp_cfg,

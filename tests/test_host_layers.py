@@ -138,7 +138,10 @@ def test_tensor_ownership_of_fused_and_in_place_shortcuts():
     # ResNet-50: sixteen fused convolutions; in place, every stage shares one tensor from its first block's output on
     kinds = lambda n: [n.layer_info(i)["kind"] for i in range(n.num_layers)]
     net = Network(zoo.resnet50_cfg(2, fuse_shortcut=True), device=-1)
-    assert sum(net.output_writer(i) != i for i in range(net.num_layers)) == 16
+    own = [i for i, k in enumerate(kinds(net)) if k not in ("cost_layer", "dropout_layer")]
+    assert sum(net.output_writer(i) != i for i in own) == 16
+    cost = net.num_layers - 1          # the closing [cost] layer has no tensor: it reports its producer, the softmax layer
+    assert kinds(net)[cost] == "cost_layer" and net.output_writer(cost) == cost - 1
     net = Network(zoo.resnet50_cfg(2, fuse_shortcut=True, in_place=True), device=-1)
     sc = [i for i, k in enumerate(kinds(net)) if k == "shortcut_layer"]
     assert [net.output_writer(i) for i in sc] == [13, 13, 13, 29, 29, 29, 29, 53, 53, 53, 53, 53, 53, 65, 65, 65]
