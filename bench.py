@@ -243,6 +243,11 @@ def memory_bound_kernels(args, emit=True):
         for _ in range(args.warmup):
             launch()
         ctx.sync()
+        t_ramp = time.perf_counter()         # sustained clock: keep the device busy for 20 ms before timing
+        while (time.perf_counter() - t_ramp) * 1e3 < min(args.ramp_ms, 20.0):
+            for _ in range(20):
+                launch()
+            ctx.sync()
         ctx.timer_start()
         for _ in range(args.steps):
             launch()
@@ -446,6 +451,16 @@ def run_network(name, args, steps, warmup, cpu_sample):
     for _ in range(max(warmup - 1, 0)):
         net.forward()
     net.sync()
+    # Clock ramp: after an idle moment the device takes some 100 ms of work to reach its sustained clock, and W passes
+    # of a small workload are over long before that (AlexNet's first layer alone at batch 32: 74 us per launch in the
+    # first milliseconds, 65 us sustained).  Untimed passes go on until --ramp-ms of work have gone by.
+    ramp_passes = 0
+    t_ramp = time.perf_counter()
+    while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+        for _ in range(8):
+            net.forward()
+        net.sync()
+        ramp_passes += 8
     # timed region: K forward passes, synchronised on both sides; HIP events on the library's own stream
     net.timer_start()
     t0 = time.perf_counter()
@@ -572,7 +587,7 @@ def run_network(name, args, steps, warmup, cpu_sample):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": text, "batch": batch, "weights": "random-init (seeded), inference batchnorm folded",
                    "launch": "hip graph replay" if use_graph and net.graph_active else "eager",
-                   "first_pass_ms": round(first_ms, 1)},
+                   "first_pass_ms": round(first_ms, 1), "clock_ramp": "%d untimed passes (%d ms) after the %d warm-up passes" % (ramp_passes, args.ramp_ms, warmup)},
         "roofline": roofline,
     }
     if conv_layers:
@@ -616,6 +631,8 @@ def main():
     ap.add_argument("--launches", default="table", choices=["table", "search", "model"],
                     help="where convolution launches take their tile shape and k-split from: the shipped launch table (problems it does "
                          "not list are measured on first use), a fresh search of every problem, or the built-in cost model alone")
+    ap.add_argument("--ramp-ms", type=float, default=100.0, help="untimed passes run for this long after the warm-up passes, so that the timed "
+                    "passes see the device's sustained clock (0: none)")
     ap.add_argument("--dump-launches", default="", help="write the tile shape and k-split every convolution layer ran with (JSON) to this file")
     ap.add_argument("--pin-launches", default="", help="run every convolution layer with the tile shape and k-split listed in this file "
                     "(as written by --dump-launches): repeats another run's launches exactly, e.g. under counter collection")

@@ -179,12 +179,18 @@ int nbl_im2col(nbl_ctx *ctx, const float *x_dev, unsigned C, unsigned H, unsigne
  * nbl_fc_fwd: connected_layer_t::_forward_() (models/layers/connected_layer.cu:19-53; CPU twin
  * connected_layer.cc:245-277): y[B][O] = act((x[B][I] . W^T) * g + b).  (The CUDA file adds bias[0]
  * to every output, connected_layer.cu:44; the CPU file is followed.)  A plan whose fan-in is a multiple
- * of 32 holds its weights twice on the device: row-major, and as contiguous 16 KB tiles for the streaming
- * kernel. */
+ * of 32 holds its weights three times on the device: row-major, as contiguous 16 KB tiles for the tiled kernels'
+ * buffer loads, and (fan-in a multiple of 8) in operand-major order for the small-batch streaming kernel. */
 int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
                 const float *scale_host, const float *mean_host, const float *var_host,
                 unsigned I, unsigned O, int act, nbl_fc_plan **out);
 int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float *y_dev, unsigned B);
+/* Which product kernel nbl_fc_fwd runs (tests / tuning; no counterpart in the reference, whose product is cuBLAS's
+ * choice, models/layers/connected_layer.cu:27-33).  0 (default): by shape -- up to 64 rows of batch over a matrix of 24 MB
+ * or more take the weight-streaming kernel (weights from a third, operand-major copy straight into the matrix
+ * cores' operand registers, activations through LDS; needs I % 8 == 0), everything else the LDS-tiled kernels;
+ * 1: always the tiled kernels; 2: the streaming kernel wherever its shape limits allow. */
+int nbl_fc_plan_set_kernel(nbl_fc_plan *plan, int kernel);
 int nbl_fc_plan_destroy(nbl_ctx *ctx, nbl_fc_plan *plan);
 /* nbl_fc_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels, same split of the

@@ -404,6 +404,168 @@ void gemm_nt_stream_kernel(const GemmArgs a) {
     }
 }
 
+// ---- weight streaming for small batches ---------------------------------------------------------------------------
+// At up to 64 rows of batch a connected layer is one pass over its [N][K] weight matrix: 415 MB for 6.6 GFLOP in
+// VGG-16's first connected layer, so the layer lasts as long as memory takes to deliver the weights, provided nothing
+// else stands in their way.  Here the weights never touch LDS: they are stored once more in operand-major order
+// (opmajor_offset: the 64 16-byte pieces a wave's load instruction fetches for one 8-wide k block of one 32-row tile
+// are one contiguous KiB, and a tile's k blocks follow each other, so a wave reads its tile as ONE contiguous
+// stream), every lane loads its own MFMA operands straight into registers through a ring of loads per tile,
+// and no barrier sits between a weight load and its use.  Only the activations X[M][K] -- small, and shared by every
+// wave of a block -- go through LDS, a chunk of 256 k at a time, double buffered, one barrier per chunk.
+// Work split: a block is 4 waves x NT tiles of 32 neurons and one k range (blockIdx.y), FC_RING weight loads in flight
+// per tile and wave; raw sums of a split go to
+// part[blockIdx.y][M][N] for splitk_reduce_kernel, an unsplit launch applies the epilogue itself.
+constexpr int FC_KALIGN = 32;              // k ranges of blocks and the padded k extent of w_op are multiples of this many k blocks
+constexpr int FC_CHUNK_KB = 32;            // k blocks of X per LDS buffer (256 k)
+constexpr int FC_X_PITCH = FC_CHUNK_KB * 8 + 4;      // floats between rows of a chunk in LDS
+
+struct FcStreamArgs {
+    const float *x; const float *w_op; float *out;
+    const float *g; const float *b; int act, has_scale;
+    int M, N, K;
+    int K8p;                // k blocks per row tile in w_op (K / 8 rounded up to a multiple of FC_KALIGN; the padding holds zeros)
+    int ntiles;             // row tiles of 32 neurons in w_op
+    int kb_per_split;       // k blocks per blockIdx.y (a multiple of FC_KALIGN)
+    int direct;             // gridDim.y == 1: out is y and the epilogue is applied here; else out is the partial-sum workspace
+};
+
+template<int MT, int NT, int FC_RING>
+__global__ __launch_bounds__(256) void fc_stream_kernel(const FcStreamArgs a) {
+    static_assert(FC_KALIGN % FC_RING == 0 && FC_CHUNK_KB % FC_RING == 0, "groups of ring refills must tile a chunk");
+    extern __shared__ __attribute__((aligned(16))) float xs[];        // [2][32 * MT][FC_X_PITCH]
+    constexpr int ROWS = 32 * MT, XBUF = ROWS * FC_X_PITCH;
+    constexpr int XLOADS = ROWS * (FC_CHUNK_KB * 2) / 256;            // 16-byte pieces of a chunk per thread
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kb_begin = blockIdx.y * a.kb_per_split;
+    const int nkb = min(a.kb_per_split, a.K8p - kb_begin);            // > 0 and a multiple of FC_KALIGN by construction
+    const int nchunks = (nkb + FC_CHUNK_KB - 1) / FC_CHUNK_KB;
+
+    // weights: tile rt of this wave starts at byte (rt * K8p + kb_begin) * 1024; the lane's piece at + lane * 16
+    const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.w_op), 0,
+                                                                          (int)((unsigned)a.ntiles * (unsigned)a.K8p * 1024u), 0x00020000);
+    int rt[NT]; unsigned wlane[NT], wbase[NT];
+    #pragma unroll
+    for(int j = 0; j < NT; j++) {
+        rt[j] = (blockIdx.x * 4 + wave) * NT + j;
+        wlane[j] = rt[j] < a.ntiles ? (unsigned)lane * 16u : 0x80000000u;       // a tile past the matrix loads zeros and no memory
+        wbase[j] = (unsigned)(rt[j] < a.ntiles ? rt[j] : 0) * (unsigned)a.K8p * 1024u + (unsigned)kb_begin * 1024u;
+    }
+    vec4f ring[NT][FC_RING];
+    auto load_w = [&](int j, int slot, int kbl) {
+        // past the block's last k block the last one is read again (never multiplied): no branch, no new memory traffic
+        const unsigned so = wbase[j] + (unsigned)min(kbl, nkb - 1) * 1024u;
+        ring[j][slot] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(wres, (int)wlane[j], (int)so, 0));
+    };
+    #pragma unroll
+    for(int u = 0; u < FC_RING; u++)
+        #pragma unroll
+        for(int j = 0; j < NT; j++) load_w(j, u, u);
+
+    // activations: thread t stages the 16-byte pieces (row = t / 64 + 4 * i, column piece t % 64) of a chunk
+    const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.x), 0,
+                                                                          (int)((unsigned)a.M * (unsigned)a.K * 4u), 0x00020000);
+    const int xcol = tid & 63, xrow0 = tid >> 6;
+    vec4f xstage[XLOADS];
+    auto stage_load = [&](int c) {
+        const int k = (kb_begin + c * FC_CHUNK_KB) * 8 + xcol * 4;
+        const bool k_ok = k < a.K && k < (kb_begin + nkb) * 8;          // K is a multiple of 4: a piece is inside or outside as a whole
+        #pragma unroll
+        for(int i = 0; i < XLOADS; i++) {
+            const int row = xrow0 + 4 * i;
+            const unsigned off = k_ok && row < a.M ? ((unsigned)row * (unsigned)a.K + (unsigned)k) * 4u : 0x80000000u;
+            xstage[i] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(xres, (int)off, 0, 0));
+        }
+    };
+    auto stage_store = [&](int buf) {
+        #pragma unroll
+        for(int i = 0; i < XLOADS; i++)
+            *reinterpret_cast<vec4f*>(&xs[buf * XBUF + (xrow0 + 4 * i) * FC_X_PITCH + xcol * 4]) = xstage[i];
+    };
+
+    floatx16 acc[MT][NT];
+    #pragma unroll
+    for(int i = 0; i < MT; i++)
+        #pragma unroll
+        for(int j = 0; j < NT; j++)
+            #pragma unroll
+            for(int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    stage_load(0);
+    stage_store(0);
+    const int xlane = r * FC_X_PITCH + half * 4;           // this lane's operand piece of k block 0 of a chunk
+    int kbl = 0;                                            // k block of the block's range the next MFMAs consume
+    // One group of FC_RING k blocks from the chunk in LDS at xb: the group's activations first (LDS answers in order,
+    // so the first step waits for its own piece only), then per k block its MFMAs and at once the refill of the ring
+    // slots they have just read, so that a weight load is always FC_RING k blocks ahead of its use.  (Left to itself
+    // the scheduler moves all refills behind the group's last MFMA, where the next group's first MFMA waits for them.)
+    auto group = [&](const float *xb, int gi) __attribute__((always_inline)) {
+        #pragma unroll
+        for(int u0 = 0; u0 < FC_RING; u0 += 8) {
+            vec4f xv[8][MT];
+            #pragma unroll
+            for(int u = 0; u < 8; u++)
+                #pragma unroll
+                for(int i = 0; i < MT; i++) xv[u][i] = *reinterpret_cast<const vec4f*>(xb + i * 32 * FC_X_PITCH + (gi * FC_RING + u0 + u) * 8);
+            #pragma unroll
+            for(int u = 0; u < 8; u++) {
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for(int j = 0; j < NT; j++) {
+                    const vec4f w = ring[j][u0 + u];
+                    #pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        #pragma unroll
+                        for(int i = 0; i < MT; i++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u][i][e], w[e], acc[i][j], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for(int j = 0; j < NT; j++) load_w(j, u0 + u, kbl + u0 + u + FC_RING);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        kbl += FC_RING;
+    };
+    for(int c = 0; c < nchunks; c++) {
+        __syncthreads();        // chunk c is in LDS; every wave has finished reading the other buffer (chunk c - 1)
+        const float *xb = xs + (c & 1) * XBUF + xlane;
+        const int groups = min(FC_CHUNK_KB, nkb - c * FC_CHUNK_KB) / FC_RING;
+        for(int gi = 0; gi + 1 < groups; gi++) group(xb, gi);
+        // The next chunk's activations are requested before the chunk's LAST group and written to LDS behind it: the
+        // memory counter retires loads in issue order, so waiting for these loads means waiting for every older one --
+        // requested here, only the last group's refills are younger and the weight ring stays full across the wait.
+        if(c + 1 < nchunks) stage_load(c + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        group(xb, groups - 1);
+        if(c + 1 < nchunks) stage_store((c + 1) & 1);
+    }
+
+    // accumulator register e of a 32x32 tile: row (batch) 8*(e/4) + 4*(lane/32) + e%4, column (neuron) lane%32
+    float *__restrict__ out = a.out + (a.direct ? (size_t)0 : (size_t)blockIdx.y * a.M * a.N);
+    #pragma unroll
+    for(int j = 0; j < NT; j++) {
+        const int n = rt[j] * 32 + r;
+        if(n >= a.N) continue;
+        float gn = 1.0f, bn = 0.0f;
+        if(a.direct) { bn = a.b[n]; if(a.has_scale) gn = a.g[n]; }
+        #pragma unroll
+        for(int i = 0; i < MT; i++)
+            #pragma unroll
+            for(int e = 0; e < 16; e++) {
+                const int m = i * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+                if(m >= a.M) continue;
+                float v = acc[i][j][e];
+                if(a.direct) {
+                    v = a.has_scale ? v * gn + bn : v + bn;
+                    v = nbl_act_apply(a.act, v);
+                }
+                out[(size_t)m * a.N + n] = v;
+            }
+    }
+}
+
 // y[m][n] = act((sum_z part[z][m][n]) * g[n] + b[n]), the parts added in ascending z.  VEC adjacent n per thread
 // (VEC = 4 needs N % 4 == 0 and 16-byte aligned buffers); eight parts are requested before the first is added, so
 // the kernel is one memory round trip per eight parts instead of one per part.
@@ -735,6 +897,8 @@ struct nbl_fc_plan {
     unsigned I, O; int act; bool has_scale;
     float *w_dev, *g_dev, *b_dev;
     float *w_tiled_dev;         // the weights once more as contiguous 16 KB [128 rows][32 k] tiles (I % 32 == 0), or NULL
+    float *w_op_dev; unsigned K8p;      // ... and in operand-major order for fc_stream_kernel (I % 8 == 0), K8p k blocks per row tile, or NULL
+    int kernel;                 // 0: chosen per call; 1: the LDS-tiled kernels; 2: the weight-streaming kernel wherever it applies
     float *ws_dev; size_t ws_bytes;     // split-K partial sums, grown on demand
 };
 
@@ -765,13 +929,113 @@ struct nbl_rnn_plan {
 
 namespace {
 
+// Grows the plan's split-K workspace to `need` bytes (or checks the fixed one) and returns where the parts go.
+int splitk_workspace(nbl_ctx *ctx, size_t need, int S, int M, int N, float **ws, size_t *ws_bytes,
+                     float *fixed_ws, size_t fixed_cap, float **part) {
+    if(fixed_ws) {
+        if(need > fixed_cap)
+            return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: the %d partial sums of this %d x %d product need %zu bytes, "
+                            "the static scratch holds %zu", S, M, N, need, fixed_cap);
+        *part = fixed_ws;
+        return NBL_OK;
+    }
+    if(*ws_bytes < need) {
+        int rc = nbl_free(ctx, *ws);
+        *ws = NULL; *ws_bytes = 0;
+        if(rc != NBL_OK) return rc;
+        if((rc = nbl_malloc(ctx, (void**)ws, need)) != NBL_OK) return rc;
+        *ws_bytes = need;
+    }
+    *part = *ws;
+    return NBL_OK;
+}
+
+int launch_splitk_reduce(nbl_ctx *ctx, const float *part, float *C, const float *g, const float *b, int M, int N, int S,
+                         int act, int has_scale) {
+    const size_t total = (size_t)M * N;
+    if(N % 4 == 0 && aligned16(part) && aligned16(C))
+        hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
+                           part, C, g, b, M, N, S, act, has_scale);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
+                           part, C, g, b, M, N, S, act, has_scale);
+    NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
+    return NBL_OK;
+}
+
+template<int MT, int NT, int RING>
+int launch_fc_stream_kernel(nbl_ctx *ctx, const FcStreamArgs &a, dim3 grid) {
+    const size_t lds = (size_t)2 * 32 * MT * FC_X_PITCH * sizeof(float);
+    static bool raised = false;         // more than 64 KB of dynamic LDS has to be asked for, once per kernel
+    if(!raised && lds > 64 * 1024) {
+        NBL_HIP(ctx, hipFuncSetAttribute((const void*)fc_stream_kernel<MT, NT, RING>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((fc_stream_kernel<MT, NT, RING>), grid, dim3(256), lds, ctx->stream, a);
+    NBL_LAUNCH_CHECK(ctx, "fc_stream_kernel");
+    return NBL_OK;
+}
+
+// The weight-streaming kernel over operand-major weights.  Returns 1 (and launches nothing) for a shape it does not take.
+int launch_fc_stream(nbl_ctx *ctx, const float *A, const float *Bw_op, unsigned K8p, float *C, int M, int N, int K,
+                     const float *g, const float *b, int act, int has_scale, float **ws, size_t *ws_bytes,
+                     float *fixed_ws, size_t fixed_cap) {
+    const unsigned ntiles = nbl_div_up(N, 32);
+    if(M > 64 || K % 8 != 0 || (size_t)ntiles * K8p * 1024 >= (1ull << 32) || (size_t)M * K * 4 >= (1ull << 31))
+        return 1;
+    // One tile of 32 neurons per wave and 16 loads in flight: measured against two tiles per wave and rings of 8 and 32
+    // on VGG-16's connected layers at batch 32 (80.2 us against 84.0 / 82.1 / 81.7 for the 415 MB layer, 18.3 against
+    // 20.1 / 22.0 / 20.9 for the 68 MB one): the finer blocks halve the partial sums a split launch writes.
+    constexpr int NT = 1, RING = 16;
+    const int MT = M <= 32 ? 1 : 2;
+    const unsigned groups = nbl_div_up(ntiles, 4 * NT);
+    // Split of the k range: blocks are dealt to the CUs evenly, so the launch lasts as long as the CU with the most
+    // work.  In bytes a CU has to pull: its blocks' weights, a fixed cost per block (start-up: the first chunk of
+    // activations, the ring's first loads), and its share of the partial sums written and read back.
+    int best_s = 1; double best_cost = 0.0;
+    for(int s = 1; s <= 64; s++) {
+        const unsigned kbps = nbl_div_up(nbl_div_up(K8p, s), FC_KALIGN) * FC_KALIGN, s_eff = nbl_div_up(K8p, kbps);
+        if((int)s_eff != s) continue;
+        const double rounds = (double)nbl_div_up_sz((size_t)groups * s, ctx->num_cu);
+        const double cost = rounds * ((double)kbps * 4 * NT * 1024 + 48.0 * 1024) +
+                            (s > 1 ? 2.0 * s * M * N * 4 / ctx->num_cu + 64.0 * 1024 : 0.0);
+        if(s == 1 || cost < best_cost) { best_cost = cost; best_s = s; }
+    }
+    FcStreamArgs a;
+    a.x = A; a.w_op = Bw_op; a.g = g; a.b = b; a.act = act; a.has_scale = has_scale;
+    a.M = M; a.N = N; a.K = K; a.K8p = (int)K8p; a.ntiles = (int)ntiles;
+    a.kb_per_split = (int)(nbl_div_up(nbl_div_up(K8p, best_s), FC_KALIGN) * FC_KALIGN);
+    const int S = (int)nbl_div_up(K8p, a.kb_per_split);
+    a.direct = S == 1;
+    float *part = C;
+    if(S > 1) {
+        const int rc = splitk_workspace(ctx, (size_t)S * M * N * sizeof(float), S, M, N, ws, ws_bytes, fixed_ws, fixed_cap, &part);
+        if(rc != NBL_OK) return rc;
+    }
+    a.out = part;
+    const dim3 grid(groups, S);
+    const int rc = MT == 1 ? launch_fc_stream_kernel<1, NT, RING>(ctx, a, grid) : launch_fc_stream_kernel<2, NT, RING>(ctx, a, grid);
+    if(rc != NBL_OK) return rc;
+    if(S > 1) return launch_splitk_reduce(ctx, part, C, g, b, M, N, S, act, has_scale);
+    return NBL_OK;
+}
+
 // Bw_tiled: the same weights as 16 KB tiles (see GemmArgs::b_tiled), or NULL; used whenever the buffer-load kernel runs
 // ws / ws_bytes: the plan's split-K workspace, grown here on demand (NULL: never split).  With fixed_ws the partial
 // sums go to that buffer of fixed_cap bytes instead and nothing is allocated or freed: a product whose split
 // needs more than fixed_cap is refused.
+// Bw_op / K8p: the weights in operand-major order (nbl_fc_pack), or NULL; kernel: nbl_fc_plan::kernel
 int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, int N, int K,
               const float *g, const float *b, int act, int has_scale, float **ws, size_t *ws_bytes,
-              const float *Bw_tiled = NULL, float *fixed_ws = NULL, size_t fixed_cap = 0) {
+              const float *Bw_tiled = NULL, float *fixed_ws = NULL, size_t fixed_cap = 0,
+              const float *Bw_op = NULL, unsigned K8p = 0, int kernel = 0) {
+    // Small batches over a large matrix: the weight-streaming kernel.  (Below some tens of MB a layer is a few
+    // microseconds either way and the tiled kernel's finer k-split fills the chip better.)
+    if(Bw_op && M <= 64 && kernel != 1 && aligned16(A) && (ws || fixed_ws) &&
+       (kernel == 2 || (size_t)N * K * sizeof(float) >= ((size_t)24 << 20))) {
+        const int rc = launch_fc_stream(ctx, A, Bw_op, K8p, C, M, N, K, g, b, act, has_scale, ws, ws_bytes, fixed_ws, fixed_cap);
+        if(rc != 1) return rc;       // (a shape it does not take falls through to the tiled kernels)
+    }
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.A = A; a.Bw = Bw; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K; a.ldc = N;
@@ -807,23 +1071,9 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
                         (size_t)nbl_div_up(N, 128) * 128 * K * 4 < (1ull << 31);
     if(buf_ok && Bw_tiled) { a.Bw = Bw_tiled; a.b_tiled = 1; }
     if(S > 1) {
-        const size_t need = (size_t)S * M * N * sizeof(float);
-        float *part;
-        if(fixed_ws) {
-            if(need > fixed_cap)
-                return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd_noalloc: the %d partial sums of this %d x %d product need %zu bytes, "
-                                "the static scratch holds %zu", S, M, N, need, fixed_cap);
-            part = fixed_ws;
-        } else {
-            if(*ws_bytes < need) {
-                int rc = nbl_free(ctx, *ws);
-                *ws = NULL; *ws_bytes = 0;
-                if(rc != NBL_OK) return rc;
-                if((rc = nbl_malloc(ctx, (void**)ws, need)) != NBL_OK) return rc;
-                *ws_bytes = need;
-            }
-            part = *ws;
-        }
+        float *part = NULL;
+        const int rc_ws = splitk_workspace(ctx, (size_t)S * M * N * sizeof(float), S, M, N, ws, ws_bytes, fixed_ws, fixed_cap, &part);
+        if(rc_ws != NBL_OK) return rc_ws;
         a.C = part;
         if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
@@ -835,14 +1085,8 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
         else if(BM == 64)  hipLaunchKernelGGL((gemm_nt_kernel<1, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         else               hipLaunchKernelGGL((gemm_nt_kernel<2, 2, 2, 2, EPI_PARTIAL>), grid, block, 0, ctx->stream, a);
         NBL_LAUNCH_CHECK(ctx, "gemm_nt_kernel(split-k)");
-        const size_t total = (size_t)M * N;
-        if(N % 4 == 0 && aligned16(part) && aligned16(C))
-            hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)nbl_div_up_sz(total / 4, 256)), dim3(256), 0, ctx->stream,
-                               (const float*)part, C, g, b, M, N, S, act, has_scale);
-        else
-            hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)nbl_div_up_sz(total, 256)), dim3(256), 0, ctx->stream,
-                               (const float*)part, C, g, b, M, N, S, act, has_scale);
-        NBL_LAUNCH_CHECK(ctx, "splitk_reduce_kernel");
+        const int rc_red = launch_splitk_reduce(ctx, part, C, g, b, M, N, S, act, has_scale);
+        if(rc_red != NBL_OK) return rc_red;
     } else {
         if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
@@ -876,7 +1120,7 @@ int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
     if((size_t)I * O >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_pack: weight matrix too large");
     nbl_fc_plan *p = new nbl_fc_plan();
     p->I = I; p->O = O; p->act = act; p->has_scale = scale_host != NULL;
-    p->w_dev = p->g_dev = p->b_dev = p->ws_dev = p->w_tiled_dev = NULL; p->ws_bytes = 0;
+    p->w_dev = p->g_dev = p->b_dev = p->ws_dev = p->w_tiled_dev = p->w_op_dev = NULL; p->ws_bytes = 0; p->K8p = 0; p->kernel = 0;
     std::vector<float> g(O), b(O);
     nbl_fold_batchnorm(bias_host, scale_host, mean_host, var_host, O, g.data(), b.data());
     int rc;
@@ -908,14 +1152,38 @@ int nbl_fc_pack(nbl_ctx *ctx, const float *weight_host, const float *bias_host,
             return rc;
         }
     }
+    // Operand-major copy for the weight-streaming kernel (small batches): row tiles of 32 neurons, K8p k blocks of 8
+    // each (the k range padded with zeros to whole rings of loads), the 64 pieces of a k block contiguous.
+    const unsigned K8p = nbl_div_up(nbl_div_up(I, 8), FC_KALIGN) * FC_KALIGN, ntiles = nbl_div_up(O, 32);
+    if(I % 8 == 0 && (size_t)ntiles * K8p * 1024 < (1ull << 32)) {
+        std::vector<float> wop((size_t)ntiles * K8p * 256, 0.0f);
+        for(unsigned n = 0; n < O; n++) {
+            const float *src = weight_host + (size_t)n * I;
+            float *tile = wop.data() + (size_t)(n / 32) * K8p * 256 + (n % 32) * 4;
+            for(unsigned k = 0; k < I; k += 4)      // the piece of lane (half = k / 4 % 2, r = n % 32) of k block k / 8
+                memcpy(tile + (size_t)(k / 8) * 256 + ((k / 4) % 2) * 128, src + k, 4 * sizeof(float));
+        }
+        if((rc = nbl_malloc(ctx, (void**)&p->w_op_dev, wop.size() * sizeof(float))) != NBL_OK ||
+           (rc = nbl_h2d(ctx, p->w_op_dev, wop.data(), wop.size() * sizeof(float))) != NBL_OK) {
+            nbl_fc_plan_destroy(ctx, p);
+            return rc;
+        }
+        p->K8p = K8p;
+    }
     *out = p;
+    return NBL_OK;
+}
+
+int nbl_fc_plan_set_kernel(nbl_fc_plan *p, int kernel) {
+    if(!p || kernel < 0 || kernel > 2) return NBL_EINVAL;
+    p->kernel = kernel;
     return NBL_OK;
 }
 
 int nbl_fc_plan_destroy(nbl_ctx *ctx, nbl_fc_plan *p) {
     if(!ctx || !p) return NBL_EINVAL;
     nbl_free(ctx, p->w_dev); nbl_free(ctx, p->g_dev); nbl_free(ctx, p->b_dev); nbl_free(ctx, p->ws_dev);
-    nbl_free(ctx, p->w_tiled_dev);
+    nbl_free(ctx, p->w_tiled_dev); nbl_free(ctx, p->w_op_dev);
     delete p;
     return NBL_OK;
 }
@@ -928,7 +1196,7 @@ int nbl_fc_fwd(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev, float 
         return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_fc_fwd: tensors of 2^31 elements or more are not supported");
     nbl_fc_plan *p = const_cast<nbl_fc_plan*>(plan);   // the split-K workspace is a cache
     return launch_fc(ctx, x_dev, p->w_dev, y_dev, (int)B, (int)p->O, (int)p->I, p->g_dev, p->b_dev,
-                     p->act, p->has_scale ? 1 : 0, &p->ws_dev, &p->ws_bytes, p->w_tiled_dev);
+                     p->act, p->has_scale ? 1 : 0, &p->ws_dev, &p->ws_bytes, p->w_tiled_dev, NULL, 0, p->w_op_dev, p->K8p, p->kernel);
 }
 
 // ---- fully connected without allocation ----------------------------------------------------------
@@ -980,7 +1248,8 @@ int nbl_fc_fwd_noalloc(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev
     // every partial sum the reduction reads is written by this call's product kernel first, so the contents a
     // previous call left behind never show
     return launch_fc(ctx, x_dev, plan->w_dev, y_dev, (int)B, (int)plan->O, (int)plan->I, plan->g_dev, plan->b_dev,
-                     plan->act, plan->has_scale ? 1 : 0, NULL, NULL, plan->w_tiled_dev, scratch, FC_SCRATCH_BYTES);
+                     plan->act, plan->has_scale ? 1 : 0, NULL, NULL, plan->w_tiled_dev, scratch, FC_SCRATCH_BYTES,
+                     plan->w_op_dev, plan->K8p, plan->kernel);
 }
 
 // ---- LSTM ----------------------------------------------------------------------------------------

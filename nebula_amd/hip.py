@@ -69,6 +69,7 @@ SIGNATURES = {
     "nbl_fc_pack": (C.c_int, [_vp, _f32p, _f32p, _f32p, _f32p, _f32p, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_fc_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
     "nbl_fc_plan_destroy": (C.c_int, [_vp, _vp]),
+    "nbl_fc_plan_set_kernel": (C.c_int, [_vp, C.c_int]),
     "nbl_fc_fwd_noalloc": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
     "nbl_lstm_pack": (C.c_int, [_vp, _pp, _pp, _pp, _pp, _pp, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_lstm_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
@@ -391,6 +392,10 @@ class FcPlan:
         y = out if out is not None else self.ctx.empty((B, self.O))
         self.ctx.check(lib().nbl_fc_fwd(self.ctx.h, self.p, x.ptr, y.ptr, B))
         return y
+
+    def set_kernel(self, kind):
+        """0: chosen by shape, 1: the LDS-tiled kernels, 2: the weight-streaming kernel wherever it applies."""
+        self.ctx.check(lib().nbl_fc_plan_set_kernel(self.p, kind))
 
     def noalloc(self, x, out):
         """The same product through the entry point that allocates nothing (static device scratch)."""

@@ -439,6 +439,9 @@ def test_fused_residual_written_in_place(shape):
                     in_place = plan.with_shortcut(dx, dconn, "relu", out=dconn).numpy()       # the search runs here
                     launch = plan.last_launch()
                     dconn.upload(conn)
+                    # (writing to a buffer of its own is another problem to the launch table: repeat the in-place launch)
+                    plan.set_variant(launch[0])
+                    plan.set_split(launch[1] if launch[1] > 1 else 0)
                     separate = plan.with_shortcut(dx, dconn, "relu", out=dy).numpy()
                     assert plan.last_launch() == launch
                 else:

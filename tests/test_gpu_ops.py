@@ -426,6 +426,46 @@ def test_fc_matches_oracle(ctx, case):
     assert rel(got, want) <= TOL, rel(got, want)
 
 
+# the weight-streaming kernel (operand-major weights, activations through LDS) on every shape limit: one and two
+# batch tiles with ragged rows, neuron counts that leave part tiles and part blocks, fan-ins of a single k block,
+# of part rings and part chunks, unsplit and split launches; and VGG-16's two large connected layers at batch 32
+FC_STREAM = [(1, 8, 5, False, "linear"), (32, 64, 32, False, "relu"), (31, 72, 257, True, "leaky"), (33, 264, 100, False, "relu"),
+             (64, 2056, 513, True, "linear"), (17, 4096, 1000, False, "logistic"), (48, 520, 62, True, "linear"),
+             (5, 12288, 2500, False, "relu"), (32, 25088, 4096, False, "relu"), (32, 4096, 4096, True, "relu"),
+             (64, 9216, 4096, False, "relu")]
+
+
+@pytest.mark.parametrize("case", FC_STREAM)
+def test_fc_weight_streaming_kernel_matches_oracle_and_the_tiled_kernels(ctx, case):
+    announce("fc stream", case)
+    B, I, O, bn, act = case
+    rng = np.random.default_rng(B * 11 + I + O)
+    x = rng.standard_normal((B, I)).astype(np.float32)
+    w = (rng.standard_normal((O, I)) * np.sqrt(2.0 / I)).astype(np.float32)
+    b = (rng.standard_normal(O) * 0.1).astype(np.float32)
+    bnp = None
+    if bn:
+        bnp = (rng.uniform(0.8, 1.2, O).astype(np.float32), (rng.standard_normal(O) * 0.1).astype(np.float32),
+               rng.uniform(0.5, 1.5, O).astype(np.float32))
+    ob.use_openblas(threads=8)
+    want = ob.connected_forward(x, w, b, bnp, act)
+    ob.use_custom_gemm()
+    plan = ctx.fc_pack(w, b, bnp, act)
+    dx = ctx.array(x)
+    plan.set_kernel(2)
+    y = ctx.empty((B, O))
+    from nebula_amd import hip
+    ctx.check(hip.lib().nbl_lds_fill(ctx.h, 0xffffffff))     # stale LDS must not show
+    got = plan(dx, out=y).numpy()
+    assert np.isfinite(got).all()
+    assert rel(got, want) <= TOL, rel(got, want)
+    again = plan(dx).numpy()
+    np.testing.assert_array_equal(bits(again), bits(got))          # fixed summation order
+    plan.set_kernel(1)
+    tiled = plan(dx).numpy()
+    assert rel(got, tiled) <= 2e-5, rel(got, tiled)
+
+
 def test_bias_and_batchnorm_primitives(ctx):
     announce("bias/bn primitives")
     rng = np.random.default_rng(31)

@@ -66,3 +66,42 @@ def test_fc_noalloc_refuses_what_the_scratch_cannot_hold():
         # the allocating entry point takes the same call
         ref = plan(x).numpy()
         assert np.isfinite(ref).all()
+
+
+def test_fc_noalloc_inside_a_stream_capture_replays_bit_equal():
+    """The entry point is for callers that cannot allocate, a stream capture among them: captured into a HIP graph on
+    the context's own stream (nothing in the call may synchronise, allocate or look a symbol up), then replayed several
+    times with eager work of the same context between the replays; every replay must give nbl_fc_fwd's bits."""
+    import ctypes as C
+    from nebula_amd import hip
+    rt = C.CDLL("libamdhip64.so")
+    rng = np.random.default_rng(79)
+    I, O, B = 4096, 1000, 48
+    w = (rng.standard_normal((O, I)) * np.sqrt(2.0 / I)).astype(np.float32)
+    b = (rng.standard_normal(O) * 0.1).astype(np.float32)
+    with hip.Ctx(0) as ctx:
+        plan = ctx.fc_pack(w, b, None, "relu")
+        xs = [rng.standard_normal((B, I)).astype(np.float32) for _ in range(3)]
+        dx = ctx.array(xs[0])
+        want = [plan(ctx.array(x)).numpy() for x in xs]
+        out = ctx.empty((B, O))
+        stream = C.c_void_p(hip.lib().nbl_ctx_stream(ctx.h))
+        ctx.sync()
+        graph, graph_exec = C.c_void_p(), C.c_void_p()
+        assert rt.hipStreamBeginCapture(stream, C.c_int(1)) == 0          # hipStreamCaptureModeThreadLocal
+        rc = hip.lib().nbl_fc_fwd_noalloc(ctx.h, plan.p, dx.ptr, out.ptr, B)
+        end = rt.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0, hip.lib().nbl_last_error(ctx.h)
+        assert end == 0 and graph.value
+        assert rt.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, C.c_size_t(0)) == 0
+        try:
+            for n, which in enumerate((0, 1, 2, 1)):
+                print("CASE fc_noalloc graph replay", n, flush=True)
+                dx.upload(xs[which])                                      # eager work of the program between replays
+                ctx.check(hip.lib().nbl_fill_zero(ctx.h, out.ptr, out.nbytes))
+                assert rt.hipGraphLaunch(graph_exec, stream) == 0
+                ctx.sync()
+                np.testing.assert_array_equal(bits(out.numpy()), bits(want[which]))
+        finally:
+            rt.hipGraphExecDestroy(graph_exec)
+            rt.hipGraphDestroy(graph)
