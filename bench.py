@@ -240,6 +240,8 @@ def memory_bound_kernels(args, emit=True):
     out = []
 
     def timed(name, nbytes, launch, note=""):
+        if args.only and args.only not in name:
+            return
         for _ in range(args.warmup):
             launch()
         ctx.sync()
@@ -332,11 +334,14 @@ def memory_bound_kernels(args, emit=True):
     # weight-streaming connected layers (the whole layer: product, split-K reduction, bias, relu)
     for name, B_, I, O in (("VGG-16 fc6", 32, 25088, 4096), ("AlexNet fc6", 128, 9216, 4096), ("VGG-16 fc7", 32, 4096, 4096),
                            ("LSTM projection (last step)", 64, 1024, 10000)):
+        label = "connected %s  %d x %d -> %d" % (name, B_, I, O)
+        if args.only and args.only not in label:
+            continue
         w = (rng.standard_normal((O, 8)).astype(np.float32) * 0.01).repeat(I // 8, axis=1)
         plan = ctx.fc_pack(w, np.zeros(O, np.float32), None, "relu")
         del w
         x = rand((B_, I)); y = ctx.empty((B_, O))
-        timed("connected %s  %d x %d -> %d" % (name, B_, I, O), 4 * (I * O + B_ * I + B_ * O), lambda: plan(x, out=y))
+        timed(label, 4 * (I * O + B_ * I + B_ * O), lambda: plan(x, out=y))
         # a product with more FLOP per byte than the machine balance (157.3 TFLOP/s over 8 TB/s) is bound by the matrix pipe
         out[-1]["flop_per_byte"] = round(2.0 * B_ * I * O / out[-1]["bytes"], 1)
         out[-1]["matrix_bound"] = out[-1]["flop_per_byte"] > PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
@@ -347,7 +352,8 @@ def memory_bound_kernels(args, emit=True):
         r["launch_bound"] = r["bytes"] < (64 << 20)
     if not emit:
         return out
-    worst = min(r["frac_of_8TBps"] for r in out[1:] if not r["launch_bound"] and not r.get("matrix_bound"))
+    rated = [r["frac_of_8TBps"] for r in (out if args.only else out[1:]) if not r["launch_bound"] and not r.get("matrix_bound")]
+    worst = min(rated) if rated else None
     print(json.dumps({"metric": "memory-bound kernels, fraction of the 8 TB/s HBM peak (lowest of the kernels that move 64 MB or more and are not matrix-bound)", "value": worst,
                       "unit": "fraction", "steps": args.steps, "warmup": args.warmup, "peak_GBps": PEAK_HBM_GBS, "kernels": out}), flush=True)
 
@@ -625,6 +631,7 @@ def main():
     ap.add_argument("--conv-split", type=int, default=-1, help="k-split mode of --workload conv (-1 launch table or search, 0 off, 1 model)")
     ap.add_argument("--conv-residual", type=int, default=0, help="1: --workload conv adds a same-shape residual and relu in the epilogue (fused shortcut)")
     ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--only", default="", help="--workload memops: time only the kernels whose label contains this text (counter passes over one kernel)")
     ap.add_argument("--cpu-sample", type=int, default=-1, help="images in the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--recurrent-net", default="lstm", choices=["lstm", "rnn"], help="network of --workload ptb")
