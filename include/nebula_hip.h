@@ -209,7 +209,7 @@ int nbl_fc_fwd_noalloc(nbl_ctx *ctx, const nbl_fc_plan *plan, const float *x_dev
  * scale/mean/var_host are arrays of eight [H] vectors, or NULL when batch_normalize=0.
  * sub_act is the [lstm] section's activation, which the reference applies inside every sub-layer.
  * nbl_lstm_fwd: lstm_layer_t::_forward_() (models/layers/lstm_layer.cu:15-140; CPU twin
- * lstm_layer.cc:233-346) from zero hidden and cell state: x_dev [T][B][I] -> y_dev [T][B][H].
+ * lstm_layer.cc:233-346) from zero hidden and cell state (or a kept one, below): x_dev [T][B][I] -> y_dev [T][B][H].
  * The per-step 8 GEMMs + 5 saxpy + 7 copies + 7 elementwise kernels become one input-side GEMM over
  * all steps and one fused recurrent kernel per step.  cell_dev (optional, may be NULL) receives the
  * final cell state [B][H]. */
@@ -218,6 +218,22 @@ int nbl_lstm_pack(nbl_ctx *ctx, const float *const *weight_host, const float *co
                   unsigned I, unsigned H, int sub_act, nbl_lstm_plan **out);
 int nbl_lstm_fwd(nbl_ctx *ctx, nbl_lstm_plan *plan, const float *x_dev, float *y_dev, float *cell_dev,
                  unsigned T, unsigned B);
+/* State kept between passes.  lstm_layer_t never clears hidden_state and cell_state between forward() calls
+ * (lstm_layer.cu:15-140: the buffers are written in every step and read again by step 0 of the next call), which
+ * is how the reference's recurrent driver runs one long token stream as consecutive batches of time_steps.  Its
+ * two paths disagree on what exactly is kept (the .cu re-reads slot 0 of its per-step cell buffer, i.e. the cell
+ * state after the FIRST step of the previous call, beside the last hidden state; the .cc does not rewind its
+ * sub-layers at all), so this library offers the recurrence's own state and leaves the choice to the caller:
+ * nbl_lstm_plan_carry_state(on = 1): from now on a pass starts from h_T and c_T of the previous pass of the same
+ *   plan when that pass had the same B (otherwise, and always with on = 0, the default, from zero).  Passes of
+ *   T1 and T2 steps then give what one pass of T1 + T2 steps gives (to rounding: the input-side product of a pass
+ *   is one matrix product over all its steps, whose summation order may depend on their number).
+ * nbl_lstm_plan_reset_state: the next pass starts from zero (a new sequence); carrying stays on.
+ * nbl_lstm_plan_set_state: the next pass with this B starts from h_dev, c_dev ([B][H] each, copied on the
+ *   context's stream); the plan must be carrying.  The state a pass ended with is its y[T-1] and cell_dev. */
+int nbl_lstm_plan_carry_state(nbl_ctx *ctx, nbl_lstm_plan *plan, int on);
+int nbl_lstm_plan_reset_state(nbl_ctx *ctx, nbl_lstm_plan *plan);
+int nbl_lstm_plan_set_state(nbl_ctx *ctx, nbl_lstm_plan *plan, const float *h_dev, const float *c_dev, unsigned B);
 /* The same layer fed by the recurrent driver's one-hot rows (models/networks/recurrent.cc:179-204, one 1.0
  * per row of input_size = vocabulary entries), given as the position of that 1: tokens_dev[T*B], time-major.
  * The input-side product  x . U^T  is then a gather of T*B columns of U (rows of a transposed copy the plan

@@ -104,6 +104,13 @@ int nbl_net_softmax_copy(nbl_net *net, int enabled);
  * nbl_net_graph_active: 1 while passes are replays of a recorded graph, 0 otherwise (also when recording was
  * not possible and the network stayed eager). */
 int nbl_net_set_graph(nbl_net *net, int enabled);
+/* enabled = 1 (also the [net] key carry_state=1, which the reference ignores): every [lstm] layer starts a pass
+ * from the hidden and cell state its previous pass ended with (nbl_lstm_plan_carry_state), as the reference's
+ * layers do between the batches of one token stream (lstm_layer.cu:15-140 never clears them); the default starts
+ * every pass from zero.  Passes of a carrying network are never recorded into a HIP graph (what a pass reads
+ * depends on the pass before it).  nbl_net_reset_state: the next pass starts from zero again (a new stream). */
+int nbl_net_set_carry_state(nbl_net *net, int enabled);
+int nbl_net_reset_state(nbl_net *net);
 int nbl_net_graph_active(nbl_net *net);
 /* the nbl_ctx* of the network (include/nebula_hip.h), e.g. for nbl_timer_start/stop */
 void *nbl_net_ctx(nbl_net *net);

@@ -914,6 +914,9 @@ struct nbl_lstm_plan {
     float *part_dev; size_t part_bytes;   // split-K partial sums of one recurrent step
     float *ucat_t_dev;                    // [I][4*Hp] transpose of ucat_dev, built on the first token-input forward
     unsigned G;                           // gate interleave: row of (gate, h) = (h/G)*4G + gate*G + h%G; 8 = single-launch steps
+    // hidden and cell state kept between forward passes (hidden_state / cell_state of lstm_layer_t, which its forward
+    // never clears): carry != 0 starts a pass from the state the previous pass of the same batch size ended with
+    int carry; unsigned state_B;          // state_B: batch size the kept state belongs to, 0 = none (start from zero)
 };
 
 // rnn_layer_t: three connected sub-layers (input, hidden, output gate) and the per-forward buffers
@@ -1336,6 +1339,41 @@ int nbl_lstm_plan_destroy(nbl_ctx *ctx, nbl_lstm_plan *p) {
     return NBL_OK;
 }
 
+// h [B][H] row-major -> the operand-major copy lstm_step_kernel reads (rows past B stay as they are)
+__global__ __launch_bounds__(256)
+void lstm_state_to_opmajor_kernel(const float *__restrict__ h, float *__restrict__ hop, unsigned B, unsigned H) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if(i >= (size_t)B * H) return;
+    const unsigned m = (unsigned)(i / H), k = (unsigned)(i % H);
+    hop[opmajor_offset(m, k, H)] = h[i];
+}
+
+// Buffers of the running state for batch size B (grown on demand; growing drops a kept state).
+static int lstm_state_buffers(nbl_ctx *ctx, nbl_lstm_plan *p, unsigned B) {
+    int rc;
+    const size_t st_need = (size_t)B * p->H * sizeof(float);
+    if(p->state_bytes < st_need) {
+        if((rc = nbl_free(ctx, p->h0_dev)) != NBL_OK || (rc = nbl_free(ctx, p->c_dev)) != NBL_OK) return rc;
+        p->h0_dev = p->c_dev = NULL; p->state_bytes = 0; p->state_B = 0;
+        if((rc = nbl_malloc(ctx, (void**)&p->h0_dev, st_need)) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->c_dev, st_need)) != NBL_OK) return rc;
+        p->state_bytes = st_need;
+    }
+    const size_t hop_need = (size_t)nbl_div_up(B, 32) * 32 * p->H * sizeof(float);
+    if(p->G == 8 && p->hop_bytes < hop_need) {
+        if((rc = nbl_free(ctx, p->hop_dev[0])) != NBL_OK || (rc = nbl_free(ctx, p->hop_dev[1])) != NBL_OK) return rc;
+        p->hop_dev[0] = p->hop_dev[1] = NULL; p->hop_bytes = 0; p->state_B = 0;
+        if((rc = nbl_malloc(ctx, (void**)&p->hop_dev[0], hop_need)) != NBL_OK ||
+           (rc = nbl_malloc(ctx, (void**)&p->hop_dev[1], hop_need)) != NBL_OK) return rc;
+        p->hop_bytes = hop_need;
+        // rows past the batch are read (their sums are dropped) and must hold numbers; the step kernel writes
+        // real rows only, so zeroing once is enough
+        if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK ||
+           (rc = nbl_fill_zero(ctx, p->hop_dev[1], hop_need)) != NBL_OK) return rc;
+    }
+    return NBL_OK;
+}
+
 // x_dev: dense input rows, or NULL with tokens_dev: one token per row (one-hot input)
 static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, const unsigned *tokens_dev, float *y_dev,
                         float *cell_dev, unsigned T, unsigned B) {
@@ -1351,29 +1389,17 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
         if((rc = nbl_malloc(ctx, (void**)&p->gx_dev, gx_need)) != NBL_OK) return rc;
         p->gx_bytes = gx_need;
     }
-    if(p->state_bytes < st_need) {
-        if((rc = nbl_free(ctx, p->h0_dev)) != NBL_OK || (rc = nbl_free(ctx, p->c_dev)) != NBL_OK) return rc;
-        p->h0_dev = p->c_dev = NULL; p->state_bytes = 0;
-        if((rc = nbl_malloc(ctx, (void**)&p->h0_dev, st_need)) != NBL_OK ||
-           (rc = nbl_malloc(ctx, (void**)&p->c_dev, st_need)) != NBL_OK) return rc;
-        p->state_bytes = st_need;
-    }
-    // zero initial hidden and cell state (first forward() of a fresh reference layer)
-    if((rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK) return rc;
+    if((rc = lstm_state_buffers(ctx, p, B)) != NBL_OK) return rc;
     const size_t hop_need = (size_t)nbl_div_up(B, 32) * 32 * p->H * sizeof(float);
-    if(p->G == 8) {
-        if(p->hop_bytes < hop_need) {
-            if((rc = nbl_free(ctx, p->hop_dev[0])) != NBL_OK || (rc = nbl_free(ctx, p->hop_dev[1])) != NBL_OK) return rc;
-            p->hop_dev[0] = p->hop_dev[1] = NULL; p->hop_bytes = 0;
-            if((rc = nbl_malloc(ctx, (void**)&p->hop_dev[0], hop_need)) != NBL_OK ||
-               (rc = nbl_malloc(ctx, (void**)&p->hop_dev[1], hop_need)) != NBL_OK) return rc;
-            p->hop_bytes = hop_need;
-            // rows past the batch are read (their sums are dropped) and must hold numbers; the step kernel writes
-            // real rows only, so zeroing once is enough for the buffer step 0 writes
-            if((rc = nbl_fill_zero(ctx, p->hop_dev[1], hop_need)) != NBL_OK) return rc;
-        }
-        if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK) return rc;      // h_{-1} = 0
-    } else if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK) return rc;
+    // Initial state: zero (the first forward() of a fresh reference layer), or -- when the plan carries its state and
+    // holds one for this batch size -- h and c as the previous pass (or nbl_lstm_plan_set_state) left them:
+    // c in c_dev, h in hop_dev[0] (operand-major) or h0_dev.
+    if(!(p->carry && p->state_B == B)) {
+        if((rc = nbl_fill_zero(ctx, p->c_dev, st_need)) != NBL_OK) return rc;
+        if(p->G == 8) { if((rc = nbl_fill_zero(ctx, p->hop_dev[0], hop_need)) != NBL_OK) return rc; }
+        else if((rc = nbl_fill_zero(ctx, p->h0_dev, st_need)) != NBL_OK) return rc;
+    }
+    p->state_B = 0;       // (set again once this pass has been queued completely)
     // input half for every step at once: gx[T*B][Np] = sub_act(x . Ucat^T + bu)
     if(tokens_dev) {
         if(!p->ucat_t_dev) {
@@ -1448,6 +1474,43 @@ static int lstm_forward(nbl_ctx *ctx, nbl_lstm_plan *p, const float *x_dev, cons
     }
     if(cell_dev)
         NBL_HIP(ctx, hipMemcpyAsync(cell_dev, p->c_dev, st_need, hipMemcpyDeviceToDevice, ctx->stream));
+    // The state a carrying plan starts its next pass from: c is in c_dev already; h_T is the buffer the last step
+    // wrote (operand-major), or a copy of y[T-1] (the caller may overwrite y before the next pass).
+    if(p->G == 8) { if(T & 1) std::swap(p->hop_dev[0], p->hop_dev[1]); }
+    else if(p->carry) NBL_HIP(ctx, hipMemcpyAsync(p->h0_dev, y_dev + (size_t)(T - 1) * step, st_need, hipMemcpyDeviceToDevice, ctx->stream));
+    p->state_B = B;
+    return NBL_OK;
+}
+
+int nbl_lstm_plan_carry_state(nbl_ctx *ctx, nbl_lstm_plan *p, int on) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p != NULL, "nbl_lstm_plan_carry_state: NULL plan");
+    if(!on || !p->carry) p->state_B = 0;       // a state left by a pass that did not keep h is not a state to start from
+    p->carry = on != 0;
+    return NBL_OK;
+}
+
+int nbl_lstm_plan_reset_state(nbl_ctx *ctx, nbl_lstm_plan *p) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p != NULL, "nbl_lstm_plan_reset_state: NULL plan");
+    p->state_B = 0;
+    return NBL_OK;
+}
+
+int nbl_lstm_plan_set_state(nbl_ctx *ctx, nbl_lstm_plan *p, const float *h_dev, const float *c_dev, unsigned B) {
+    if(!ctx) return NBL_EINVAL;
+    NBL_REQUIRE(ctx, p && h_dev && c_dev && B > 0, "nbl_lstm_plan_set_state: NULL argument or empty batch");
+    NBL_REQUIRE(ctx, p->carry, "nbl_lstm_plan_set_state: the plan does not carry state (nbl_lstm_plan_carry_state)");
+    int rc;
+    if((rc = lstm_state_buffers(ctx, p, B)) != NBL_OK) return rc;
+    const size_t st = (size_t)B * p->H * sizeof(float);
+    NBL_HIP(ctx, hipMemcpyAsync(p->c_dev, c_dev, st, hipMemcpyDeviceToDevice, ctx->stream));
+    if(p->G == 8) {
+        hipLaunchKernelGGL(lstm_state_to_opmajor_kernel, dim3(nbl_div_up((unsigned)((size_t)B * p->H), 256)), dim3(256), 0, ctx->stream,
+                           h_dev, p->hop_dev[0], B, p->H);
+        NBL_LAUNCH_CHECK(ctx, "lstm_state_to_opmajor_kernel");
+    } else NBL_HIP(ctx, hipMemcpyAsync(p->h0_dev, h_dev, st, hipMemcpyDeviceToDevice, ctx->stream));
+    p->state_B = B;
     return NBL_OK;
 }
 

@@ -73,6 +73,9 @@ SIGNATURES = {
     "nbl_fc_fwd_noalloc": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
     "nbl_lstm_pack": (C.c_int, [_vp, _pp, _pp, _pp, _pp, _pp, _u, _u, C.c_int, C.POINTER(_vp)]),
     "nbl_lstm_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u, _u]),
+    "nbl_lstm_plan_carry_state": (C.c_int, [_vp, _vp, C.c_int]),
+    "nbl_lstm_plan_reset_state": (C.c_int, [_vp, _vp]),
+    "nbl_lstm_plan_set_state": (C.c_int, [_vp, _vp, _vp, _vp, _u]),
     "nbl_lstm_plan_destroy": (C.c_int, [_vp, _vp]),
     "nbl_pool_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _u, _u, _u, _u, _u, _u, _u, C.c_int]),
     "nbl_pool_out_dim": (_u, [_u, _u, _u]),
@@ -427,6 +430,17 @@ class LstmPlan:
         y = out if out is not None else self.ctx.empty((T, B, self.H))
         self.ctx.check(lib().nbl_lstm_fwd(self.ctx.h, self.p, x.ptr, y.ptr, cell.ptr if cell is not None else None, T, B))
         return y
+
+    def carry_state(self, on=True):
+        """Start every pass from the state the previous pass of the same batch size ended with (off: from zero)."""
+        self.ctx.check(lib().nbl_lstm_plan_carry_state(self.ctx.h, self.p, 1 if on else 0))
+
+    def reset_state(self):
+        self.ctx.check(lib().nbl_lstm_plan_reset_state(self.ctx.h, self.p))
+
+    def set_state(self, h, c):
+        """h, c: DeviceArrays [B][H], the state the next pass of that batch size starts from."""
+        self.ctx.check(lib().nbl_lstm_plan_set_state(self.ctx.h, self.p, h.ptr, c.ptr, h.shape[0]))
 
     def from_tokens(self, tokens, out=None, cell=None):
         """tokens: DeviceArray [T][B] of uint32, the positions of the 1s of one-hot input rows."""

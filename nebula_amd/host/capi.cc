@@ -246,6 +246,14 @@ int nbl_net_set_graph(nbl_net *n, int enabled) {
     return 0;
 }
 
+int nbl_net_set_carry_state(nbl_net *n, int enabled) {
+    NBL_NET_TRY(if(!n) throw std::runtime_error("NULL argument"); n->net->set_carry_state(enabled != 0));
+}
+
+int nbl_net_reset_state(nbl_net *n) {
+    NBL_NET_TRY(if(!n) throw std::runtime_error("NULL argument"); n->net->reset_state());
+}
+
 int nbl_net_graph_active(nbl_net *n) { return n ? (n->net->graph_active() ? 1 : 0) : -1; }
 
 void *nbl_net_ctx(nbl_net *n) { return n ? (void*)n->net->ctx : NULL; }

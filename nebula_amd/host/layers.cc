@@ -533,6 +533,15 @@ void lstm_layer_t::pack() {
               nbl_lstm_pack(network->ctx, w, b, batch_normalize ? sc : NULL, batch_normalize ? mu : NULL,
                             batch_normalize ? var : NULL, input_size, output_size, (int)activation_type, &plan),
               "nbl_lstm_pack");
+    carry_state(network->carry_state);
+}
+
+void lstm_layer_t::carry_state(bool on) {
+    if(plan) nbl_check(network->ctx, nbl_lstm_plan_carry_state(network->ctx, plan, on ? 1 : 0), "nbl_lstm_plan_carry_state");
+}
+
+void lstm_layer_t::reset_state() {
+    if(plan) nbl_check(network->ctx, nbl_lstm_plan_reset_state(network->ctx, plan), "nbl_lstm_plan_reset_state");
 }
 
 // network->batch_size counts every (time step, sequence) row; rows are time-major.

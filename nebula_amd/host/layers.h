@@ -201,6 +201,9 @@ public:
     void store_weight(std::fstream &m_weight_file);
     void _forward_();
     void weight_fields(std::vector<weight_field_t> &out) const;
+    // hidden_state / cell_state between forward() calls (network_t::carry_state): kept, or cleared for a new stream
+    void carry_state(bool on);
+    void reset_state();
 private:
     void pack();
     bool batch_normalize;

@@ -24,7 +24,7 @@ network_t::network_t() :
     run_type(UNDEFINED_RUN), num_threads(1),
     learning_rate(0.001f), momentum(0.9f), decay(0.0001f), cost(0.0f),
     input_height(1), input_width(1), input_channel(1), input_size(0), batch_size(1), time_step(1),
-    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1), pool_index(false), defer_host_copy(false),
+    input_data(NULL), input_label(NULL), input_data_dev(NULL), ctx(NULL), input_tokens_dev(NULL), conv_split(-1), pool_index(false), carry_state(false), defer_host_copy(false),
     input_layer(NULL), output_layer(NULL), num_layers(0) {}
 
 network_t::~network_t() {}
@@ -136,6 +136,7 @@ void inference_net_t::build(config_t &config) {
                 sc.get_setting("input_size", &input_size);
                 sc.get_setting("time_steps", &time_step);
                 sc.get_setting("last_step_only", &last_step_only);
+                sc.get_setting("carry_state", &carry_state);
                 batch_size *= time_step;                 // rows = time steps x sequences, time-major
             }
             if(!batch_size || !input_size) throw std::runtime_error("Error: [net] gives an empty input");
@@ -346,6 +347,17 @@ void inference_net_t::forward_eager() {
     for(unsigned i = 0; i < num_layers; i++) run_layer(i);
 }
 
+void inference_net_t::set_carry_state(bool on) {
+    carry_state = on;
+    for(size_t i = 0; i < layers.size(); i++)
+        if(layers[i]->layer_type == LSTM_LAYER) static_cast<lstm_layer_t*>(layers[i])->carry_state(on);
+}
+
+void inference_net_t::reset_state() {
+    for(size_t i = 0; i < layers.size(); i++)
+        if(layers[i]->layer_type == LSTM_LAYER) static_cast<lstm_layer_t*>(layers[i])->reset_state();
+}
+
 void inference_net_t::invalidate_graph() {
     ++graph_epoch;
     if(graph_exec) {
@@ -370,7 +382,7 @@ unsigned long long inference_net_t::pass_key() const {
 
 void inference_net_t::forward() {
     if(!ctx) throw std::runtime_error("Error: no device (dry-run network)");
-    if(!use_graph || graph_unusable) { forward_eager(); return; }
+    if(!use_graph || graph_unusable || carry_state) { forward_eager(); return; }
     hipStream_t stream = (hipStream_t)nbl_ctx_stream(ctx);
     const unsigned long long key = pass_key();
     if(graph_exec && key != graph_key) invalidate_graph();      // (bumps the epoch: the key is taken again below)

@@ -58,6 +58,8 @@ public:
     // reference's forward writes for its backward pass (models/layers/pooling_layer.cc:132,140).  Inference never
     // reads it, so by default it is neither allocated nor written (a third of a max-pool's memory traffic).
     bool pool_index;
+    // [net] key `carry_state=1` (see inference_net_t::set_carry_state): [lstm] layers keep their state between passes
+    bool carry_state;
     // Set while inference_net_t::forward() records or replays a HIP graph: a layer that copies to the host queues
     // the copy on the stream instead of waiting for it, and forward() waits once at its end.
     bool defer_host_copy;
@@ -132,6 +134,11 @@ public:
     // what a pass launches (weights, token vs. dense input, last_step_only, the softmax copy) makes the next
     // pass start over; call invalidate_graph() after changing a layer behind the network's back.
     bool use_graph;
+    // [net] key `carry_state=1` of a recurrent net (a key the reference ignores): [lstm] layers start a pass from the
+    // hidden and cell state their previous pass ended with, as lstm_layer_t's never-cleared hidden_state / cell_state
+    // do between the batches of one token stream; reset_state() starts a new stream.  Such passes run eagerly.
+    void set_carry_state(bool on);
+    void reset_state();
     void invalidate_graph();
     bool graph_active() const { return graph_exec != NULL; }   // true once a recorded pass is being replayed
     void forward_eager();

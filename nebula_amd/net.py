@@ -42,6 +42,8 @@ SIGNATURES = {
     "nbl_net_conv_problem": (C.c_int, [_vp, C.c_int, C.POINTER(_u)]),
     "nbl_net_softmax_copy": (C.c_int, [_vp, C.c_int]),
     "nbl_net_set_graph": (C.c_int, [_vp, C.c_int]),
+    "nbl_net_set_carry_state": (C.c_int, [_vp, C.c_int]),
+    "nbl_net_reset_state": (C.c_int, [_vp]),
     "nbl_net_graph_active": (C.c_int, [_vp]),
     "nbl_net_ctx": (_vp, [_vp]),
 }
@@ -218,6 +220,14 @@ class Network:
     def set_graph(self, enabled):
         """Record one forward pass into a HIP graph and replay it from then on (first pass eager, second recorded)."""
         lib().nbl_net_set_graph(self.h, 1 if enabled else 0)
+
+    def set_carry_state(self, enabled):
+        """[lstm] layers start a pass from the state their previous pass ended with (also [net] carry_state=1)."""
+        self._check(lib().nbl_net_set_carry_state(self.h, 1 if enabled else 0))
+
+    def reset_state(self):
+        """The next pass of a carrying network starts from zero state again (a new token stream)."""
+        self._check(lib().nbl_net_reset_state(self.h))
 
     @property
     def graph_active(self):

@@ -216,6 +216,59 @@ def test_lstm_last_step_only_against_oracle():
             np.testing.assert_array_equal(probs.argmax(1), want[3].argmax(1))
 
 
+@pytest.mark.parametrize("H", [128, 48])
+def test_lstm_network_carries_state_between_batches_of_one_stream(H):
+    """The reference's recurrent driver runs a token stream as consecutive batches of time_steps and its LSTM layers
+    never clear their state in between (lstm_layer.cu:15-140).  [net] carry_state=1: two passes over the halves of a
+    sequence give what the oracle gives for the whole sequence; reset_state starts a new stream; the default network
+    starts every pass from zero."""
+    from nebula_amd import zoo
+    from nebula_amd.net import Network
+    print("CASE lstm network carry_state", H, flush=True)
+    T, B, I, Cn = 6, 5, 24, 19
+    rng = np.random.default_rng(H)
+    whole_cfg = zoo.lstm_cfg(batch=B, time_steps=T, input_size=I, hidden=H, layers=2, classes=Cn)
+    half_cfg = zoo.lstm_cfg(batch=B, time_steps=T // 2, input_size=I, hidden=H, layers=2, classes=Cn)
+    onet = ob.OracleNet(whole_cfg)
+    blob = np.concatenate([rng.uniform(-1, 1, int(np.prod(sh))).astype(np.float32) / np.float32(np.sqrt(H))
+                           for _, _, sh in ob.weight_layout(onet.specs)])
+    onet.load_weights(blob)
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    ob.use_custom_gemm()
+    want = onet.forward(x)
+    half_rows = T // 2 * B
+    ohalf = ob.OracleNet(half_cfg)
+    ohalf.load_weights(blob)
+    want_fresh = ohalf.forward(x[T // 2:])               # the second half from zero state
+    with Network(half_cfg.replace("[net]\n", "[net]\ncarry_state=1\nhip_graph=1\n", 1)) as net:
+        net.load_weight_blob(blob)
+        for rep in range(2):
+            parts = []
+            for part in (x[:T // 2], x[T // 2:]):
+                net.set_input(part)
+                net.forward()
+                parts.append([net.output(i).copy() for i in range(4)])
+            assert not net.graph_active                   # what a pass reads depends on the pass before it
+            for i in (0, 1, 3):
+                w = want[i].reshape(T * B, -1)
+                assert rel(parts[0][i].reshape(half_rows, -1), w[:half_rows]) <= TOL, (rep, i)
+                assert rel(parts[1][i].reshape(half_rows, -1), w[half_rows:]) <= TOL, (rep, i)
+            assert rel(parts[1][1], want_fresh[1].ravel()) > 1e-3          # (the state does matter for these weights)
+            net.reset_state()
+        net.set_carry_state(False)
+        net.set_input(x[T // 2:])
+        net.forward()
+        assert rel(net.output(1), want_fresh[1].ravel()) <= TOL
+        net.forward()
+        assert rel(net.output(1), want_fresh[1].ravel()) <= TOL
+    with Network(half_cfg) as net:                          # the default: every pass from zero
+        net.load_weight_blob(blob)
+        for _ in range(2):
+            net.set_input(x[T // 2:])
+            net.forward()
+            assert rel(net.output(3).reshape(half_rows, -1), want_fresh[3]) <= TOL
+
+
 def test_fused_shortcut_is_bit_identical():
     """fuse_shortcut=1 moves the residual add into the convolution's epilogue: same operations, same order."""
     from nebula_amd.net import Network

@@ -538,6 +538,59 @@ def test_lstm_matches_oracle(ctx, case):
     np.testing.assert_array_equal(bits(got2), bits(got))
 
 
+# (T1, T2, B, I, H): hidden sizes of the one-launch-per-step kernel with odd and even pass lengths (its two state
+# buffers swap roles after an odd pass), of the split-K path and of the single fused kernel
+LSTM_CARRY = [(3, 4, 5, 48, 256), (2, 2, 37, 64, 128), (1, 1, 33, 32, 384), (3, 2, 6, 64, 96), (2, 3, 7, 20, 33)]
+
+
+@pytest.mark.parametrize("case", LSTM_CARRY)
+def test_lstm_state_kept_between_passes(ctx, case):
+    """lstm_layer_t never clears hidden_state / cell_state between forward() calls (lstm_layer.cu:15-140).  A carrying
+    plan run on the two parts of a sequence must give what one pass over the whole sequence gives (and what the oracle
+    gives for the whole sequence); reset_state and a different batch size start from zero; set_state on a second
+    plan continues from y[T1-1] and the cell state the first pass returned."""
+    announce("lstm carry", case)
+    T1, T2, B, I, H = case
+    T = T1 + T2
+    rng = np.random.default_rng(T * 100 + B + I + H)
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    names = ("iW", "fW", "oW", "cW", "iU", "fU", "oU", "cU")
+    wt = [(rng.uniform(-1, 1, (H, H if n[1] == "W" else I)) / np.sqrt(H)).astype(np.float32) for n in names]
+    bs = [(rng.uniform(-1, 1, H) / np.sqrt(H)).astype(np.float32) for n in names]
+    want, wcell = ob.lstm_forward(x, wt, bs, None, "linear", want_cell=True)
+    plan = ctx.lstm_pack(wt, bs, None, "linear")
+    whole = plan(ctx.array(x)).numpy()
+    assert rel(whole, want) <= TOL
+    plan.carry_state(True)
+    cell1, cell2 = ctx.empty((B, H)), ctx.empty((B, H))
+    first = plan(ctx.array(x[:T1]), cell=cell1).numpy()
+    second = plan(ctx.array(x[T1:]), cell=cell2).numpy()
+    assert rel(first, whole[:T1]) <= 1e-5 and rel(second, whole[T1:]) <= 1e-5, (rel(first, whole[:T1]), rel(second, whole[T1:]))
+    assert rel(second, want[T1:]) <= TOL and rel(cell2.numpy(), wcell[-1]) <= TOL
+    # a third pass goes on from the second: the same as the oracle run on the sequence with its first part repeated
+    third = plan(ctx.array(x[:T1])).numpy()
+    want3 = ob.lstm_forward(np.concatenate([x, x[:T1]]), wt, bs, None, "linear")
+    assert rel(third, want3[T:]) <= TOL
+    # a new stream, a pass of another batch size, and carrying switched off all start from zero
+    plan.reset_state()
+    np.testing.assert_array_equal(bits(plan(ctx.array(x[:T1])).numpy()), bits(first))
+    if B > 1:
+        fewer = plan(ctx.array(np.ascontiguousarray(x[:T1, :B - 1]))).numpy()
+        assert rel(fewer, want[:T1, :B - 1]) <= TOL
+        again = plan(ctx.array(x[:T1])).numpy()                      # the kept state belongs to B - 1 rows: not used
+        np.testing.assert_array_equal(bits(again), bits(first))
+    plan.carry_state(False)
+    np.testing.assert_array_equal(bits(plan(ctx.array(x[:T1])).numpy()), bits(first))
+    np.testing.assert_array_equal(bits(plan(ctx.array(x[:T1])).numpy()), bits(first))
+    # the state handed over explicitly to another plan of the same weights
+    other = ctx.lstm_pack(wt, bs, None, "linear")
+    with pytest.raises(Exception):
+        other.set_state(ctx.array(first[-1]), cell1)          # not carrying: refused
+    other.carry_state(True)
+    other.set_state(ctx.array(first[-1]), cell1)
+    np.testing.assert_array_equal(bits(other(ctx.array(x[T1:])).numpy()), bits(second))
+
+
 @pytest.mark.parametrize("H", [128, 33])
 def test_lstm_token_input_equals_one_hot_input(ctx, H):
     """One-hot input rows given as token indices: the gather must reproduce the dense product bit for bit."""

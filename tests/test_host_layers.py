@@ -145,3 +145,14 @@ def test_tensor_ownership_of_fused_and_in_place_shortcuts():
     net = Network(zoo.resnet50_cfg(2, fuse_shortcut=True, in_place=True), device=-1)
     sc = [i for i, k in enumerate(kinds(net)) if k == "shortcut_layer"]
     assert [net.output_writer(i) for i in sc] == [13, 13, 13, 29, 29, 29, 29, 53, 53, 53, 53, 53, 53, 65, 65, 65]
+
+
+def test_carry_state_key_and_calls_on_a_dry_run_network():
+    """[net] carry_state=1 is parsed for recurrent nets; the state calls are harmless before weights exist and on
+    networks without [lstm] layers."""
+    cfg = zoo.lstm_cfg(batch=2, time_steps=3, input_size=8, hidden=16, layers=2, classes=5)
+    for text in (cfg, cfg.replace("[net]\n", "[net]\ncarry_state=1\n", 1), zoo.alexnet_cfg(1)):
+        with dry(text) as net:
+            net.set_carry_state(True)
+            net.reset_state()
+            net.set_carry_state(False)
