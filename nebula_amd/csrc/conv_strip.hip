@@ -275,10 +275,10 @@ int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *
     const size_t grid = nbl_div_up_sz((size_t)a.runs, 64) * 64 * a.tiles_m;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     const bool fast = sp->act == NBL_ACT_RELU || sp->act == NBL_ACT_LINEAR || sp->act == NBL_ACT_LEAKY || sp->act == NBL_ACT_RELIE;
-    // more than 64 KB of dynamic LDS has to be asked for, once per kernel
+    // more than 64 KB of dynamic LDS has to be asked for, once per kernel and device
 #define NBL_STRIP_LAUNCH(MT, FA) \
-    do { static bool raised = false; \
-         if(!raised) { NBL_HIP(ctx, hipFuncSetAttribute((const void*)conv_strip_kernel<MT, FA>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)STRIP_LDS_LIMIT)); raised = true; } \
+    do { static nbl_lds_limit_raised raised; \
+         NBL_HIP(ctx, raised.ensure(conv_strip_kernel<MT, FA>, ctx->device, (int)STRIP_LDS_LIMIT)); \
          hipLaunchKernelGGL((conv_strip_kernel<MT, FA>), dim3((unsigned)grid), dim3(256), sp->lds_bytes, ctx->stream, a); } while(0)
     if(sp->mt == 2)      { if(fast) NBL_STRIP_LAUNCH(2, true); else NBL_STRIP_LAUNCH(2, false); }
     else if(sp->mt == 3) { if(fast) NBL_STRIP_LAUNCH(3, true); else NBL_STRIP_LAUNCH(3, false); }

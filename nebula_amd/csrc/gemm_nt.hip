@@ -969,11 +969,8 @@ int launch_splitk_reduce(nbl_ctx *ctx, const float *part, float *C, const float 
 template<int MT, int NT, int RING>
 int launch_fc_stream_kernel(nbl_ctx *ctx, const FcStreamArgs &a, dim3 grid) {
     const size_t lds = (size_t)2 * 32 * MT * FC_X_PITCH * sizeof(float);
-    static bool raised = false;         // more than 64 KB of dynamic LDS has to be asked for, once per kernel
-    if(!raised && lds > 64 * 1024) {
-        NBL_HIP(ctx, hipFuncSetAttribute((const void*)fc_stream_kernel<MT, NT, RING>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        raised = true;
-    }
+    static nbl_lds_limit_raised raised;         // more than 64 KB of dynamic LDS has to be asked for, once per kernel and device
+    if(lds > 64 * 1024) NBL_HIP(ctx, raised.ensure(fc_stream_kernel<MT, NT, RING>, ctx->device, (int)lds));
     hipLaunchKernelGGL((fc_stream_kernel<MT, NT, RING>), grid, dim3(256), lds, ctx->stream, a);
     NBL_LAUNCH_CHECK(ctx, "fc_stream_kernel");
     return NBL_OK;
@@ -1033,9 +1030,11 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
               const float *Bw_tiled = NULL, float *fixed_ws = NULL, size_t fixed_cap = 0,
               const float *Bw_op = NULL, unsigned K8p = 0, int kernel = 0) {
     // Small batches over a large matrix: the weight-streaming kernel.  (Below some tens of MB a layer is a few
-    // microseconds either way and the tiled kernel's finer k-split fills the chip better.)
+    // microseconds either way and the tiled kernel's finer k-split fills the chip better; so it does for a short
+    // fan-in, which leaves a streaming block two or three chunks of activations to walk: the 1024 -> 10000
+    // projection behind an LSTM at batch 64 takes 23.5 us tiled and 26.1 us streamed, a fan-in of 4096 ties.)
     if(Bw_op && M <= 64 && kernel != 1 && aligned16(A) && (ws || fixed_ws) &&
-       (kernel == 2 || (size_t)N * K * sizeof(float) >= ((size_t)24 << 20))) {
+       (kernel == 2 || ((size_t)N * K * sizeof(float) >= ((size_t)24 << 20) && K >= 4096))) {
         const int rc = launch_fc_stream(ctx, A, Bw_op, K8p, C, M, N, K, g, b, act, has_scale, ws, ws_bytes, fixed_ws, fixed_cap);
         if(rc != 1) return rc;       // (a shape it does not take falls through to the tiled kernels)
     }

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -42,6 +43,24 @@ int nbl_fail(nbl_ctx *ctx, int code, const char *fmt, ...);
     do { hipError_t e_ = hipGetLastError(); \
          if(e_ != hipSuccess) return nbl_fail((ctx), NBL_EHIP, "launch of %s failed: %s", what, \
                                               hipGetErrorString(e_)); } while(0)
+
+// A kernel that asks for more than 64 KB of dynamic LDS must have that limit raised first, on every device it runs
+// on (hipFuncSetAttribute acts on the current device).  One of these per kernel remembers which devices are done:
+// one bit per device ordinal, ordinals from 64 on are asked for every time.
+struct nbl_lds_limit_raised {
+    std::atomic<unsigned long long> devices{0};
+    template<typename Kernel>
+    hipError_t ensure(Kernel kernel, int device, int bytes) {
+        if(device >= 0 && device < 64 && (devices.load(std::memory_order_acquire) >> device & 1)) return hipSuccess;
+        int current = -1;
+        hipError_t e = hipGetDevice(&current);
+        if(e == hipSuccess && current != device) e = hipSetDevice(device);
+        if(e == hipSuccess) e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if(current >= 0 && current != device) (void)hipSetDevice(current);
+        if(e == hipSuccess && device >= 0 && device < 64) devices.fetch_or(1ull << device, std::memory_order_release);
+        return e;
+    }
+};
 
 static inline unsigned nbl_div_up(unsigned a, unsigned b) { return (a + b - 1) / b; }
 static inline size_t nbl_div_up_sz(size_t a, size_t b) { return (a + b - 1) / b; }
