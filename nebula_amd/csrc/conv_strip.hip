@@ -39,6 +39,7 @@ struct StripArgs {
     int act;
     int runs;               // pixel tiles of the launch (tiles_per_image * batch)
     FastDiv div_tiles_m, div_tiles_per_image, div_ow;      // the block's set-up divides by these three
+    FastDiv div_rows;       // staging: line -> channel
 };
 
 // (MT = 2: five blocks per CU fit its LDS use when the registers allow it too -- 6272 tiles of the 7x7 stem at batch 64
@@ -68,39 +69,39 @@ void conv_strip_kernel(const StripArgs a) {
     const int oh0 = (int)a.div_ow.div((unsigned)p0), ih0 = oh0 * a.stride - a.pad;
 
     // ---- stage the strip: rows ih0 .. ih0 + rows - 1, columns -pad .. W + pad - 1 of every channel ----
-    // One (channel, row) line per wave at a time, lanes along the line, through a buffer descriptor that covers
+    // The strip's (channel, row) lines are dealt to the four waves in turn, lanes along the line, through a buffer descriptor that covers
     // exactly that image row: a column left or right of the image is an out-of-range offset and reads 0, a row
     // above or below the image gets an empty descriptor.  Per element that leaves one load, one LDS write and the
     // add for its LDS address -- ordinary vector instructions are paid for in matrix-pipe time.  STAGE_LINES lines
     // are requested before the first is written, so a block waits for memory a few times, not once per line.
     {
-        constexpr int STAGE_LINES = 4, STAGE_J = 4;          // lines in flight per wave; 64-lane pieces of a line
+        constexpr int STAGE_LINES = 8, STAGE_J = 4;          // lines in flight per wave; 64-lane pieces of a line
         const float *__restrict__ xim = a.x + (size_t)img * a.C * a.H * a.W;
+        const int nlines = a.C * a.rows;                     // line l = (channel l / rows, row l % rows); wave w takes lines w, w + 4, ...
         for(int w0 = 0; w0 < a.pitch; w0 += 64 * STAGE_J) {                                     // (one pass unless a row has more than 256 columns)
             unsigned voff[STAGE_J];                          // the range check looks at this per-lane offset only
             #pragma unroll
             for(int j = 0; j < STAGE_J; j++) voff[j] = (unsigned)(w0 + lane + 64 * j - a.pad) * 4u;   // wraps (out of range) left of the image
-            for(int c = 0; c < a.C; c++) {
-                for(int r0 = wave; r0 < a.rows; r0 += 4 * STAGE_LINES) {                        // rows r0, r0 + 4, ... of channel c
-                    float v[STAGE_LINES][STAGE_J];
+            for(int l0 = wave; l0 < nlines; l0 += 4 * STAGE_LINES) {
+                float v[STAGE_LINES][STAGE_J];
+                #pragma unroll
+                for(int u = 0; u < STAGE_LINES; u++) {
+                    const int l = l0 + 4 * u;                                                   // uniform
+                    const int c = (int)a.div_rows.div((unsigned)l), ih = ih0 + l - c * a.rows;
+                    const bool row_inside = l < nlines && (unsigned)ih < (unsigned)a.H;
+                    const __amdgpu_buffer_rsrc_t row = __builtin_amdgcn_make_buffer_rsrc(
+                        const_cast<float*>(xim + (row_inside ? (size_t)c * a.H + ih : 0) * a.W), 0, row_inside ? a.W * 4 : 0, 0x00020000);
                     #pragma unroll
-                    for(int u = 0; u < STAGE_LINES; u++) {
-                        const int ih = ih0 + r0 + 4 * u;                                        // uniform
-                        const bool row_inside = r0 + 4 * u < a.rows && (unsigned)ih < (unsigned)a.H;
-                        const __amdgpu_buffer_rsrc_t row = __builtin_amdgcn_make_buffer_rsrc(
-                            const_cast<float*>(xim + ((size_t)c * a.H + (row_inside ? ih : 0)) * a.W), 0, row_inside ? a.W * 4 : 0, 0x00020000);
+                    for(int j = 0; j < STAGE_J; j++)
+                        v[u][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(row, (int)voff[j], 0, 0));
+                }
+                #pragma unroll
+                for(int u = 0; u < STAGE_LINES; u++) {
+                    const int l = l0 + 4 * u;
+                    if(l < nlines) {
+                        float *dst = strip + l * a.pitch + w0 + lane;
                         #pragma unroll
-                        for(int j = 0; j < STAGE_J; j++)
-                            v[u][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(row, (int)voff[j], 0, 0));
-                    }
-                    #pragma unroll
-                    for(int u = 0; u < STAGE_LINES; u++) {
-                        const int r = r0 + 4 * u;
-                        if(r < a.rows) {
-                            float *dst = strip + (c * a.rows + r) * a.pitch + w0 + lane;
-                            #pragma unroll
-                            for(int j = 0; j < STAGE_J; j++) if(w0 + lane + 64 * j < a.pitch) dst[64 * j] = v[u][j];
-                        }
+                        for(int j = 0; j < STAGE_J; j++) if(w0 + lane + 64 * j < a.pitch) dst[64 * j] = v[u][j];
                     }
                 }
             }
@@ -271,7 +272,7 @@ int nbl_conv_strip_forward(nbl_ctx *ctx, const nbl_strip_plan *sp, const float *
     a.rows = sp->rows; a.pitch = sp->pitch; a.act = sp->act;
     a.runs = a.tiles_per_image * (int)B;
     a.div_tiles_m = make_fastdiv((unsigned)a.tiles_m); a.div_tiles_per_image = make_fastdiv((unsigned)a.tiles_per_image);
-    a.div_ow = make_fastdiv((unsigned)a.OW);
+    a.div_ow = make_fastdiv((unsigned)a.OW); a.div_rows = make_fastdiv((unsigned)a.rows);
     const size_t grid = nbl_div_up_sz((size_t)a.runs, 64) * 64 * a.tiles_m;
     if(grid >= (1ull << 31)) return nbl_fail(ctx, NBL_EUNSUPPORTED, "nbl_conv2d_fwd: grid too large");
     const bool fast = sp->act == NBL_ACT_RELU || sp->act == NBL_ACT_LINEAR || sp->act == NBL_ACT_LEAKY || sp->act == NBL_ACT_RELIE;
