@@ -1,12 +1,14 @@
 """Measures the convolution launches of the shipped networks on the device and writes the launch table.
 
-    python -m nebula_amd.tune [--out nebula_amd/launch_tables/gfx950.txt] [--rounds 3] [--workloads resnet50,vgg16,...]
+    python -m nebula_amd.tune [--out nebula_amd/launch_tables/gfx950.txt] [--rounds 3] [--workloads resnet50,vgg16,...] [--merge]
 
 Every round empties the in-memory table, builds each network at the batch size it is benchmarked at and runs one
 forward pass, which measures every convolution problem the table does not hold (nbl_conv2d_fwd's tile search) and
 enters the winner.  A problem's final entry is the choice most rounds agreed on (ties: the one with the lowest
 measured time), so a single noisy search does not decide a layer.  The file it writes is what libnebula_hip.so
 reads on first use; a network of one's own is added by running it once and calling nbl_launch_table_save.
+--merge keeps every entry the output file already holds and adds only problems it does not list (the benchmarked
+networks' entries, which the committed profiles were taken with, then stay as they are).
 """
 import argparse
 import collections
@@ -33,6 +35,14 @@ WORKLOADS = collections.OrderedDict([
     ("resnet50_fused", (lambda: zoo.resnet50_cfg(64, fuse_shortcut=True), "he")),
     ("resnet50_plain", (lambda: zoo.resnet50_cfg(64), "he")),
 ])
+# the same networks at other batch sizes (not benchmarked; listed so that a first pass at these sizes measures nothing)
+for _b in (16, 32, 128, 256):
+    WORKLOADS["resnet50_b%d" % _b] = ((lambda b=_b: zoo.resnet50_cfg(b, fuse_shortcut=True, in_place=True)), "he")
+for _b in (16, 64, 128):
+    WORKLOADS["vgg16_b%d" % _b] = ((lambda b=_b: zoo.vgg16_cfg(b)), "he")
+for _b in (32, 64, 256, 512):
+    WORKLOADS["alexnet_b%d" % _b] = ((lambda b=_b: zoo.alexnet_cfg(b)), "he")
+BENCHMARKED = ["conv1", "alexnet", "vgg16", "resnet50", "resnet50_fused", "resnet50_plain"]
 
 
 def read_table(path):
@@ -83,7 +93,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default=os.path.join(hip.PKG, "launch_tables", "gfx950.txt"))
     ap.add_argument("--rounds", type=int, default=3)
-    ap.add_argument("--workloads", default=",".join(WORKLOADS))
+    ap.add_argument("--workloads", default=",".join(BENCHMARKED), help="any of: " + ", ".join(WORKLOADS))
+    ap.add_argument("--merge", action="store_true", help="keep the entries the output file already holds; add new problems only")
     args = ap.parse_args()
     names = [n for n in args.workloads.split(",") if n]
     log = lambda *a: print(*a, file=sys.stderr, flush=True)
@@ -99,8 +110,14 @@ def main():
         tied = [c for c, n in count.items() if n == best_n]
         pick = min(tied, key=lambda c: min(us for t, s, us in seen if (t, s) == c))
         entries[key] = (pick[0], pick[1], min(us for t, s, us in seen if (t, s) == pick))
+    note = "%d rounds over %s" % (args.rounds, ", ".join(names))
+    if args.merge and os.path.exists(args.out):
+        kept = read_table(args.out)
+        log("kept %d problems of %s, %d new" % (len(kept), args.out, len(set(entries) - set(kept))))
+        entries.update(kept)
+        note = "benchmarked networks first; then, merged, " + note
     os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
-    write_table(args.out, entries, "%d rounds over %s" % (args.rounds, ", ".join(names)))
+    write_table(args.out, entries, note)
     log("wrote %d problems to %s" % (len(entries), args.out))
 
 

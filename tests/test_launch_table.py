@@ -60,7 +60,11 @@ def test_malformed_file_is_refused_with_its_line_number(tmp_path, bad):
 WORKLOADS = {"conv1": lambda: zoo.conv1_pool_cfg(32), "alexnet": lambda: zoo.alexnet_cfg(128), "vgg16": lambda: zoo.vgg16_cfg(32),
              "resnet50 (benchmarked: fused shortcuts written in place)": lambda: zoo.resnet50_cfg(64, fuse_shortcut=True, in_place=True),
              "resnet50 (fused)": lambda: zoo.resnet50_cfg(64, fuse_shortcut=True),
-             "resnet50 (as the reference's cfg reads)": lambda: zoo.resnet50_cfg(64)}
+             "resnet50 (as the reference's cfg reads)": lambda: zoo.resnet50_cfg(64),
+             # other batch sizes the table lists (not benchmarked)
+             "resnet50 batch 32": lambda: zoo.resnet50_cfg(32, fuse_shortcut=True, in_place=True),
+             "resnet50 batch 256": lambda: zoo.resnet50_cfg(256, fuse_shortcut=True, in_place=True),
+             "vgg16 batch 64": lambda: zoo.vgg16_cfg(64), "alexnet batch 256": lambda: zoo.alexnet_cfg(256)}
 
 
 @pytest.mark.parametrize("name", sorted(WORKLOADS))
