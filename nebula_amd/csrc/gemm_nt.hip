@@ -1045,8 +1045,16 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     a.g = g; a.b = b; a.act = act; a.has_scale = has_scale;
     // tile: 32*MT rows of batch per wave row
     const bool small_m = M <= 32;
-    const int BM = small_m ? 32 : (M <= 64 ? 64 : 128);
-    const int BN = 128;
+    // Large batches: 128x128 tiles hold two blocks of four waves per CU, whose stalls (tile hand-over: LDS writes, barrier,
+    // first LDS reads) tend to fall together; 64x64 tiles hold four blocks per CU and keep the matrix pipe busier
+    // wherever they alone fill the chip at least twice over without a k-split: the LSTM's input product over all
+    // time steps ([4096 x 1024].[1024 x 4096]) 277 -> 253 us.  Launches that need a k-split to fill the chip keep
+    // the large tile (AlexNet's 9216 -> 4096 layer at batch 128: 85.1 us against 86.7).
+    const bool t64 = M > 64 && a.vec_ok && K % GEMM_BK == 0 && (size_t)M * K * 4 < (1ull << 31) &&
+                     (size_t)nbl_div_up(N, 128) * 128 * K * 4 < (1ull << 31) &&
+                     (size_t)nbl_div_up(M, 64) * nbl_div_up(N, 64) >= 2 * (size_t)ctx->num_cu;
+    const int BM = t64 ? 64 : small_m ? 32 : (M <= 64 ? 64 : 128);
+    const int BN = t64 ? 64 : 128;
     const unsigned gm = nbl_div_up(M, BM), gn = nbl_div_up(N, BN);
     // Split K so that every CU walks about the same number of k-tiles: blocks are dealt to the CUs round robin, so a
     // launch lasts as long as the CU with the most blocks, ceil(blocks / CUs) chunks of k-tiles plus a partial tile
@@ -1071,13 +1079,14 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
     // every k-tile whole and both operands addressable by 31-bit byte offsets: the buffer-load variant
     const bool buf_ok = a.vec_ok && K % GEMM_BK == 0 && (size_t)M * K * 4 < (1ull << 31) &&
                         (size_t)nbl_div_up(N, 128) * 128 * K * 4 < (1ull << 31);
-    if(buf_ok && Bw_tiled) { a.Bw = Bw_tiled; a.b_tiled = 1; }
+    if(buf_ok && Bw_tiled && !t64) { a.Bw = Bw_tiled; a.b_tiled = 1; }
     if(S > 1) {
         float *part = NULL;
         const int rc_ws = splitk_workspace(ctx, (size_t)S * M * N * sizeof(float), S, M, N, ws, ws_bytes, fixed_ws, fixed_cap, &part);
         if(rc_ws != NBL_OK) return rc_ws;
         a.C = part;
-        if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
+        if(t64)                        hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 2, 2, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(buf_ok)                hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_PARTIAL, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 32 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_PARTIAL, false>), grid, block, 0, ctx->stream, a);
@@ -1090,7 +1099,8 @@ int launch_fc(nbl_ctx *ctx, const float *A, const float *Bw, float *C, int M, in
         const int rc_red = launch_splitk_reduce(ctx, part, C, g, b, M, N, S, act, has_scale);
         if(rc_red != NBL_OK) return rc_red;
     } else {
-        if(BM == 32 && buf_ok)         hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
+        if(t64)                        hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 2, 2, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
+        else if(BM == 32 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 64 && buf_ok)    hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 1, 1, 4, 4, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
         else if(buf_ok)                hipLaunchKernelGGL((gemm_nt_stream_kernel<2, 2, 2, 2, 2, EPI_DIRECT, true>), grid, block, 0, ctx->stream, a);
         else if(BM == 32 && a.vec_ok)  hipLaunchKernelGGL((gemm_nt_stream_kernel<1, 1, 1, 4, 4, EPI_DIRECT, false>), grid, block, 0, ctx->stream, a);

@@ -406,7 +406,10 @@ FC = [(7, 60, 11, False, "linear"), (32, 512, 1000, False, "relu"), (64, 2048, 1
       (1, 256, 64, False, "tanh"),
       # small batches stream the weight matrix: ragged k tails, neuron tails, one and two batch tiles, split and unsplit
       (32, 2500, 2000, False, "relu"), (64, 25088, 96, True, "relu"), (17, 1500, 1000, False, "logistic"),
-      (48, 500, 62, True, "linear"), (64, 260, 33, False, "relu"), (2, 49152, 40, False, "relu")]
+      (48, 500, 62, True, "linear"), (64, 260, 33, False, "relu"), (2, 49152, 40, False, "relu"),
+      # large batches whose 64x64 tiles alone fill the chip twice over: fan-ins of two and three k-tiles (shorter than
+      # the kernel's ring of four), ragged rows and neurons, and a square product
+      (600, 64, 3500, False, "relu"), (520, 96, 4000, True, "leaky"), (1024, 1024, 2048, False, "linear")]
 
 
 @pytest.mark.parametrize("case", FC)
